@@ -1,0 +1,44 @@
+// Host/device helpers shared by the kernels and the C ABI.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/fbfft_amd.h"
+
+namespace fbfft_amd {
+
+// real [B][h][w]; strides in floats
+struct RealView {
+  float* data;
+  int sb, sy, sx;
+  int B, h, w;
+};
+
+// complex-as-float [B][rows][cols][2]; strides in floats, (re, im) adjacent
+struct CplxView {
+  float* data;
+  int sb, sr, sc;
+  int B, rows, cols;
+};
+
+// the unsigned-compare bounds test of MemoryAccess.cuh:19-25
+__host__ __device__ __forceinline__ bool inWindow(int y, int x, int padU, int padL, int h, int w) {
+  return (unsigned)(y - padU) < (unsigned)h && (unsigned)(x - padL) < (unsigned)w;
+}
+
+inline int ceilDiv(int a, int b) { return (a + b - 1) / b; }
+
+inline bool aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
+
+inline int launchStatus() {
+  return hipPeekAtLastError() == hipSuccess ? FBFFT_SUCCESS : FBFFT_HIP_ERROR;
+}
+
+// kernel launchers implemented in the .hip files (return an fbfft_error)
+int launchFft2dSmallForward(int N, const RealView& real, const CplxView& cplx, int padL, int padU,
+                            hipStream_t s);
+int launchFft2dSmallInverse(int N, const CplxView& cplx, const RealView& real, int padL, int padU,
+                            hipStream_t s);
+
+}  // namespace fbfft_amd

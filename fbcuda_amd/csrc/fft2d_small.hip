@@ -1,0 +1,344 @@
+// 2D real-to-complex / complex-to-real transforms for N in {8, 16, 32}
+// (replaces fbfft2DVertical_{8,16,32} / fbifft2DVertical_{8,16,32},
+// fbfft/FFT2D32.cuh:361-533).  Output layout cplx[b][ky][kx], ky = 0..N/2.
+//
+// Design (one wave64 per workgroup, no workgroup-wide synchronisation):
+//   * T = N/2 lanes share a plane, so a wave carries P = 128/N planes.
+//   * column pass: lane l owns columns 2l and 2l+1.  It loads them with 8-byte
+//     loads (a wave instruction covers whole 4N-byte rows), runs two N/2-point
+//     complex FFTs on the even/odd-row packing entirely in VGPRs and applies the
+//     real-input fix-up; spectral rows 0 and N/2 (both real) travel packed as
+//     one complex row.
+//   * padded LDS transpose (row stride N + pad complex) hands lane l the whole
+//     packed row l, 16 bytes per access.
+//   * row pass: one N-point complex FFT per lane, again fully in VGPRs;
+//     bit reversal is just register naming.
+//   * the result goes back through LDS and leaves as one contiguous stream of
+//     16-byte stores per wave; rows 0 and N/2 are unpacked on the way out.
+// The inverse runs the same steps backwards.  Each plane crosses HBM exactly
+// once in each direction: 4N^2 + 8N(N/2+1) bytes.
+#include "common.h"
+#include "fft_regs.h"
+
+namespace fbfft_amd {
+namespace {
+
+template <int N>
+struct SmallCfg {
+  static constexpr int H = N / 2;
+  static constexpr int T = N / 2;          // lanes per plane
+  static constexpr int P = 64 / T;         // planes per wave
+  static constexpr int ROWS = H + 1;       // spectral rows kept in LDS
+  static constexpr int RS = N + 2;         // LDS row stride (complex): 16-byte aligned rows,
+                                           // consecutive rows start 4 (mod 64) banks apart
+  static constexpr int PS = ROWS * RS + (N == 8 ? 2 : 0);  // LDS plane stride (complex)
+  static constexpr int F4_PER_PLANE = ROWS * N / 2;        // float4 per spectrum plane
+  static constexpr int ITERS = P * F4_PER_PLANE / 64;      // float4 per lane per wave
+  static_assert(P * F4_PER_PLANE % 64 == 0, "copy loop must divide evenly");
+  static_assert(RS % 2 == 0 && PS % 2 == 0, "rows must stay 16-byte aligned");
+};
+
+__device__ __forceinline__ float4 ldsLoad4(const c32* p) {
+  return *reinterpret_cast<const float4*>(p);
+}
+__device__ __forceinline__ void ldsStore4(c32* p, c32 a, c32 b) {
+  *reinterpret_cast<float4*>(p) = float4{a.x, a.y, b.x, b.y};
+}
+
+// FAST_REAL: real is [B][N][N] with unit x stride, even row/batch strides,
+//            8-byte aligned base and zero padding -> 8-byte vector accesses.
+// FAST_CPLX: each spectrum plane is contiguous and 16-byte aligned.
+template <int N, bool FAST_REAL, bool FAST_CPLX>
+__global__ __launch_bounds__(64) void fft2dSmallForward(RealView real, CplxView cplx, int padL,
+                                                        int padU) {
+  using C = SmallCfg<N>;
+  constexpr int H = C::H, T = C::T, P = C::P, RS = C::RS, PS = C::PS;
+  __shared__ __align__(16) c32 lds[P * PS];
+
+  const int lane = threadIdx.x;
+  const int pl = lane / T;
+  const int l = lane % T;
+  const int b0 = blockIdx.x * P;
+  const int B = real.B;
+  const int b = min(b0 + pl, B - 1);  // tail lanes redo the last plane and skip the store
+
+  // ---- column pass ----
+  c32 z0[H], z1[H];
+  if constexpr (FAST_REAL) {
+    const float2* src = reinterpret_cast<const float2*>(real.data + (size_t)b * real.sb) + l;
+    const int rs2 = real.sy / 2;
+    staticFor<H>([&](auto jj) {
+      constexpr int j = decltype(jj)::value;
+      float2 r0 = src[(size_t)(2 * j) * rs2];
+      float2 r1 = src[(size_t)(2 * j + 1) * rs2];
+      z0[j] = c32{r0.x, r1.x};
+      z1[j] = c32{r0.y, r1.y};
+    });
+  } else {
+    const float* src = real.data + (size_t)b * real.sb;
+    const int x0 = 2 * l, x1 = 2 * l + 1;
+    auto fetch = [&](int y, int x) {
+      return inWindow(y, x, padU, padL, real.h, real.w)
+                 ? src[(size_t)(y - padU) * real.sy + (size_t)(x - padL) * real.sx] : 0.0f;
+    };
+    staticFor<H>([&](auto jj) {
+      constexpr int j = decltype(jj)::value;
+      z0[j] = c32{fetch(2 * j, x0), fetch(2 * j + 1, x0)};
+      z1[j] = c32{fetch(2 * j, x1), fetch(2 * j + 1, x1)};
+    });
+  }
+  difFFT<H, true>(z0);
+  difFFT<H, true>(z1);
+  {
+    c32 p0[H], p1[H];
+    realFixupForward<H>(z0, p0);
+    realFixupForward<H>(z1, p1);
+    c32* dst = lds + pl * PS + 2 * l;
+    staticFor<H>([&](auto rr) {
+      constexpr int r = decltype(rr)::value;
+      ldsStore4(dst + r * RS, p0[r], p1[r]);
+    });
+  }
+  __syncthreads();
+
+  // ---- row pass: lane l owns packed row l ----
+  c32 row[N];
+  {
+    const c32* src = lds + pl * PS + l * RS;
+    staticFor<N / 2>([&](auto jj) {
+      constexpr int j = decltype(jj)::value;
+      float4 v = ldsLoad4(src + 2 * j);
+      row[2 * j] = c32{v.x, v.y};
+      row[2 * j + 1] = c32{v.z, v.w};
+    });
+  }
+  difFFT<N, true>(row);
+  {
+    c32* dst = lds + pl * PS + l * RS;
+    staticFor<N / 2>([&](auto jj) {
+      constexpr int j = decltype(jj)::value;
+      ldsStore4(dst + 2 * j, row[slot<N>(2 * j)], row[slot<N>(2 * j + 1)]);
+    });
+  }
+  __syncthreads();
+
+  // ---- copy out: (H+1) x N complex per plane, rows 0 and H unpacked from packed row 0 ----
+  staticFor<C::ITERS>([&](auto tt) {
+    constexpr int t = decltype(tt)::value;
+    const int q = lane + 64 * t;
+    const int pp = q / C::F4_PER_PLANE;
+    const int rem = q % C::F4_PER_PLANE;
+    const int r = rem / (N / 2);
+    const int kx = 2 * (rem % (N / 2));
+    const c32* base = lds + pp * PS;
+    float4 v;
+    if (r == 0 || r == H) {
+      c32 a0 = base[kx], a1 = base[kx + 1];
+      c32 m0 = base[(N - kx) & (N - 1)], m1 = base[N - kx - 1];
+      if (r == 0) {
+        v = float4{0.5f * (a0.x + m0.x), 0.5f * (a0.y - m0.y), 0.5f * (a1.x + m1.x),
+                   0.5f * (a1.y - m1.y)};
+      } else {
+        v = float4{0.5f * (a0.y + m0.y), 0.5f * (m0.x - a0.x), 0.5f * (a1.y + m1.y),
+                   0.5f * (m1.x - a1.x)};
+      }
+    } else {
+      v = ldsLoad4(base + r * RS + kx);
+    }
+    const int bo = b0 + pp;
+    if (bo < B) {
+      if constexpr (FAST_CPLX) {
+        reinterpret_cast<float4*>(cplx.data + (size_t)bo * cplx.sb)[rem] = v;
+      } else {
+        float* o = cplx.data + (size_t)bo * cplx.sb + (size_t)r * cplx.sr + (size_t)kx * cplx.sc;
+        *reinterpret_cast<float2*>(o) = float2{v.x, v.y};
+        *reinterpret_cast<float2*>(o + cplx.sc) = float2{v.z, v.w};
+      }
+    }
+  });
+}
+
+template <int N, bool FAST_REAL, bool FAST_CPLX>
+__global__ __launch_bounds__(64) void fft2dSmallInverse(CplxView cplx, RealView real, int padL,
+                                                        int padU) {
+  using C = SmallCfg<N>;
+  constexpr int H = C::H, T = C::T, P = C::P, RS = C::RS, PS = C::PS;
+  __shared__ __align__(16) c32 lds[P * PS];
+
+  const int lane = threadIdx.x;
+  const int pl = lane / T;
+  const int l = lane % T;
+  const int b0 = blockIdx.x * P;
+  const int B = real.B;
+
+  // ---- copy in: natural [row][kx] order ----
+  staticFor<C::ITERS>([&](auto tt) {
+    constexpr int t = decltype(tt)::value;
+    const int q = lane + 64 * t;
+    const int pp = q / C::F4_PER_PLANE;
+    const int rem = q % C::F4_PER_PLANE;
+    const int r = rem / (N / 2);
+    const int kx = 2 * (rem % (N / 2));
+    const int bi = min(b0 + pp, B - 1);
+    float4 v;
+    if constexpr (FAST_CPLX) {
+      v = reinterpret_cast<const float4*>(cplx.data + (size_t)bi * cplx.sb)[rem];
+    } else {
+      const float* o = cplx.data + (size_t)bi * cplx.sb + (size_t)r * cplx.sr + (size_t)kx * cplx.sc;
+      float2 a = *reinterpret_cast<const float2*>(o);
+      float2 c = *reinterpret_cast<const float2*>(o + cplx.sc);
+      v = float4{a.x, a.y, c.x, c.y};
+    }
+    *reinterpret_cast<float4*>(lds + pp * PS + r * RS + kx) = v;
+  });
+  __syncthreads();
+
+  // ---- pack rows 0 and H into one complex row: Q = F0 + i*FH.  At kx = 0 only
+  // the real parts are used, as in the reference (fbfft/FFT2D32.cuh:310-316). ----
+  {
+    c32* r0 = lds + pl * PS + 2 * l;
+    const c32* rH = r0 + H * RS;
+    float4 a = ldsLoad4(r0);
+    float4 c = ldsLoad4(rH);
+    float4 q = float4{a.x - c.y, a.y + c.x, a.z - c.w, a.w + c.z};
+    if (l == 0) {
+      q.x = a.x;
+      q.y = c.x;
+    }
+    *reinterpret_cast<float4*>(r0) = q;
+  }
+  __syncthreads();
+
+  // ---- row pass (inverse) ----
+  c32 row[N];
+  {
+    const c32* src = lds + pl * PS + l * RS;
+    staticFor<N / 2>([&](auto jj) {
+      constexpr int j = decltype(jj)::value;
+      float4 v = ldsLoad4(src + 2 * j);
+      row[2 * j] = c32{v.x, v.y};
+      row[2 * j + 1] = c32{v.z, v.w};
+    });
+  }
+  difFFT<N, false>(row);
+  {
+    c32* dst = lds + pl * PS + l * RS;
+    staticFor<N / 2>([&](auto jj) {
+      constexpr int j = decltype(jj)::value;
+      ldsStore4(dst + 2 * j, row[slot<N>(2 * j)], row[slot<N>(2 * j + 1)]);
+    });
+  }
+  __syncthreads();
+
+  // ---- column pass (inverse): lane l owns columns 2l, 2l+1 ----
+  c32 p0[H], p1[H];
+  {
+    const c32* src = lds + pl * PS + 2 * l;
+    staticFor<H>([&](auto rr) {
+      constexpr int r = decltype(rr)::value;
+      float4 v = ldsLoad4(src + r * RS);
+      p0[r] = c32{v.x, v.y};
+      p1[r] = c32{v.z, v.w};
+    });
+  }
+  c32 z0[H], z1[H];
+  realFixupInverse<H>(p0, z0);
+  realFixupInverse<H>(p1, z1);
+  difFFT<H, false>(z0);
+  difFFT<H, false>(z1);
+
+  const int b = b0 + pl;
+  if (b >= B) return;
+  if constexpr (FAST_REAL) {
+    float2* dst = reinterpret_cast<float2*>(real.data + (size_t)b * real.sb) + l;
+    const int rs2 = real.sy / 2;
+    staticFor<H>([&](auto jj) {
+      constexpr int j = decltype(jj)::value;
+      c32 a = z0[slot<H>(j)], c = z1[slot<H>(j)];
+      dst[(size_t)(2 * j) * rs2] = float2{a.x, c.x};
+      dst[(size_t)(2 * j + 1) * rs2] = float2{a.y, c.y};
+    });
+  } else {
+    float* dst = real.data + (size_t)b * real.sb;
+    const int x0 = 2 * l, x1 = 2 * l + 1;
+    auto put = [&](int y, int x, float v) {
+      if (inWindow(y, x, padU, padL, real.h, real.w))
+        dst[(size_t)(y - padU) * real.sy + (size_t)(x - padL) * real.sx] = v;
+    };
+    staticFor<H>([&](auto jj) {
+      constexpr int j = decltype(jj)::value;
+      c32 a = z0[slot<H>(j)], c = z1[slot<H>(j)];
+      put(2 * j, x0, a.x);
+      put(2 * j, x1, c.x);
+      put(2 * j + 1, x0, a.y);
+      put(2 * j + 1, x1, c.y);
+    });
+  }
+}
+
+bool fastReal(int N, const RealView& r, int padL, int padU) {
+  return padL == 0 && padU == 0 && r.h == N && r.w == N && r.sx == 1 && r.sy % 2 == 0 &&
+         r.sb % 2 == 0 && aligned(r.data, 8);
+}
+
+bool fastCplx(int N, const CplxView& c) {
+  return c.sc == 2 && c.sr == 2 * N && c.sb % 4 == 0 && aligned(c.data, 16);
+}
+
+template <int N>
+int launchForward(const RealView& real, const CplxView& cplx, int padL, int padU, hipStream_t s) {
+  using C = SmallCfg<N>;
+  dim3 grid(ceilDiv(real.B, C::P)), block(64);
+  const bool fr = fastReal(N, real, padL, padU), fc = fastCplx(N, cplx);
+  if (fr && fc)
+    fft2dSmallForward<N, true, true><<<grid, block, 0, s>>>(real, cplx, padL, padU);
+  else if (fc)
+    fft2dSmallForward<N, false, true><<<grid, block, 0, s>>>(real, cplx, padL, padU);
+  else if (fr)
+    fft2dSmallForward<N, true, false><<<grid, block, 0, s>>>(real, cplx, padL, padU);
+  else
+    fft2dSmallForward<N, false, false><<<grid, block, 0, s>>>(real, cplx, padL, padU);
+  return launchStatus();
+}
+
+template <int N>
+int launchInverse(const CplxView& cplx, const RealView& real, int padL, int padU, hipStream_t s) {
+  using C = SmallCfg<N>;
+  dim3 grid(ceilDiv(real.B, C::P)), block(64);
+  const bool fr = fastReal(N, real, padL, padU), fc = fastCplx(N, cplx);
+  if (fr && fc)
+    fft2dSmallInverse<N, true, true><<<grid, block, 0, s>>>(cplx, real, padL, padU);
+  else if (fc)
+    fft2dSmallInverse<N, false, true><<<grid, block, 0, s>>>(cplx, real, padL, padU);
+  else if (fr)
+    fft2dSmallInverse<N, true, false><<<grid, block, 0, s>>>(cplx, real, padL, padU);
+  else
+    fft2dSmallInverse<N, false, false><<<grid, block, 0, s>>>(cplx, real, padL, padU);
+  return launchStatus();
+}
+
+}  // namespace
+
+int launchFft2dSmallForward(int N, const RealView& real, const CplxView& cplx, int padL, int padU,
+                            hipStream_t s) {
+  if (real.B <= 0) return FBFFT_SUCCESS;
+  switch (N) {
+    case 8: return launchForward<8>(real, cplx, padL, padU, s);
+    case 16: return launchForward<16>(real, cplx, padL, padU, s);
+    case 32: return launchForward<32>(real, cplx, padL, padU, s);
+  }
+  return FBFFT_UNSUPPORTED_SIZE;
+}
+
+int launchFft2dSmallInverse(int N, const CplxView& cplx, const RealView& real, int padL, int padU,
+                            hipStream_t s) {
+  if (real.B <= 0) return FBFFT_SUCCESS;
+  switch (N) {
+    case 8: return launchInverse<8>(cplx, real, padL, padU, s);
+    case 16: return launchInverse<16>(cplx, real, padL, padU, s);
+    case 32: return launchInverse<32>(cplx, real, padL, padU, s);
+  }
+  return FBFFT_UNSUPPORTED_SIZE;
+}
+
+}  // namespace fbfft_amd

@@ -1,0 +1,147 @@
+// In-register FFT building blocks for gfx950.
+//
+// Every transform here runs inside one lane on a small array of complex values
+// that the compiler keeps in VGPRs: all indices and all twiddle factors are
+// compile-time constants, so a butterfly is a handful of v_add/v_sub/v_fma with
+// literal operands and no cross-lane traffic.  The twiddles come from the same
+// correctly-rounded 128-entry table the reference uses (fbfft/Twiddles.cuh:322-453).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include <type_traits>
+#include <utility>
+
+namespace fbfft_amd {
+
+typedef float2 c32;
+
+constexpr uint32_t kTwiddleBits[256] = {
+#include "twiddles_f32.inc"
+};
+
+// e^{+i*pi*IDX/128}
+template <int IDX>
+struct TableEntry {
+  static_assert(IDX >= 0 && IDX < 128, "twiddle index out of range");
+  static constexpr float c = __builtin_bit_cast(float, kTwiddleBits[2 * IDX]);
+  static constexpr float s = __builtin_bit_cast(float, kTwiddleBits[2 * IDX + 1]);
+};
+
+// compile-time loop: f(std::integral_constant<int, 0>{}) ... f(<N-1>)
+template <typename F, int... Is>
+__device__ __forceinline__ void staticForImpl(F&& f, std::integer_sequence<int, Is...>) {
+  (f(std::integral_constant<int, Is>{}), ...);
+}
+template <int N, typename F>
+__device__ __forceinline__ void staticFor(F&& f) {
+  staticForImpl(static_cast<F&&>(f), std::make_integer_sequence<int, N>{});
+}
+
+constexpr int ilog2(int n) { return n <= 1 ? 0 : 1 + ilog2(n / 2); }
+
+constexpr int bitrev(int x, int bits) {
+  int r = 0;
+  for (int i = 0; i < bits; ++i) r |= ((x >> i) & 1) << (bits - 1 - i);
+  return r;
+}
+
+__device__ __forceinline__ c32 cadd(c32 a, c32 b) { return c32{a.x + b.x, a.y + b.y}; }
+__device__ __forceinline__ c32 csub(c32 a, c32 b) { return c32{a.x - b.x, a.y - b.y}; }
+__device__ __forceinline__ c32 cmul(c32 a, c32 b) {
+  return c32{a.x * b.x - a.y * b.y, a.x * b.y + a.y * b.x};
+}
+__device__ __forceinline__ c32 cconj(c32 a) { return c32{a.x, -a.y}; }
+
+// d * W, W = e^{-/+ 2*pi*i*K/M} (forward: minus), K in [0, M/2)
+template <int M, int K, bool FWD>
+__device__ __forceinline__ c32 mulRoot(c32 d) {
+  static_assert(K >= 0 && 2 * K < M, "root index");
+  if constexpr (K == 0) {
+    return d;
+  } else if constexpr (4 * K == M) {
+    return FWD ? c32{d.y, -d.x} : c32{-d.y, d.x};
+  } else if constexpr (8 * K == M) {
+    constexpr float h = TableEntry<32>::c;  // sqrt(1/2)
+    return FWD ? c32{(d.x + d.y) * h, (d.y - d.x) * h} : c32{(d.x - d.y) * h, (d.x + d.y) * h};
+  } else if constexpr (8 * K == 3 * M) {
+    constexpr float h = TableEntry<32>::c;
+    return FWD ? c32{(d.y - d.x) * h, -(d.x + d.y) * h} : c32{-(d.x + d.y) * h, (d.x - d.y) * h};
+  } else {
+    constexpr float c = TableEntry<K * 256 / M>::c;
+    constexpr float s = FWD ? -TableEntry<K * 256 / M>::s : TableEntry<K * 256 / M>::s;
+    return c32{d.x * c - d.y * s, d.x * s + d.y * c};
+  }
+}
+
+// Radix-2 decimation in frequency of a[0..N): natural order in, bit-reversed
+// order out (the value with frequency index k ends up in a[bitrev(k)]).
+template <int N, bool FWD, int M = N>
+__device__ __forceinline__ void difFFT(c32 (&a)[N]) {
+  if constexpr (M >= 2) {
+    constexpr int half = M / 2;
+    staticFor<N / M>([&](auto blk) {
+      staticFor<half>([&](auto kk) {
+        constexpr int k = decltype(kk)::value;
+        constexpr int lo = decltype(blk)::value * M + k;
+        constexpr int hi = lo + half;
+        c32 s = cadd(a[lo], a[hi]);
+        c32 d = csub(a[lo], a[hi]);
+        a[lo] = s;
+        a[hi] = mulRoot<M, k, FWD>(d);
+      });
+    });
+    difFFT<N, FWD, M / 2>(a);
+  }
+}
+
+// index of frequency k in the output of difFFT<N>
+template <int N>
+constexpr int slot(int k) {
+  return bitrev(k, ilog2(N));
+}
+
+// Forward real-input fix-up.  z (in difFFT output order) is the H-point complex
+// FFT of z[j] = x[2j] + i*x[2j+1]; on return p[k], k = 1..H-1, holds F[k] of the
+// 2H-point real transform (natural order) and p[0] = (F[0], F[H]) packed as
+// (re, im) - both are real.
+template <int H>
+__device__ __forceinline__ void realFixupForward(const c32 (&z)[H], c32 (&p)[H]) {
+  constexpr int N = 2 * H;
+  {
+    c32 z0 = z[0];
+    p[0] = c32{z0.x + z0.y, z0.x - z0.y};
+  }
+  staticFor<H - 1>([&](auto kk) {
+    constexpr int k = decltype(kk)::value + 1;
+    c32 a = z[slot<H>(k)];
+    c32 b = z[slot<H>(H - k)];
+    // E = (a + conj b)/2, O = -i (a - conj b)/2, F = E + W_N^k O
+    c32 e = c32{0.5f * (a.x + b.x), 0.5f * (a.y - b.y)};
+    c32 o = c32{0.5f * (a.y + b.y), -0.5f * (a.x - b.x)};
+    c32 wo = mulRoot<N, k, true>(o);
+    p[k] = cadd(e, wo);
+  });
+}
+
+// Inverse of realFixupForward without the 1/2 factors (gain 2): p as above
+// (natural order, p[0] packed) -> z in NATURAL order, ready for an inverse
+// H-point complex FFT whose output z[j] = (x[2j], x[2j+1]) * gain.
+template <int H>
+__device__ __forceinline__ void realFixupInverse(const c32 (&p)[H], c32 (&z)[H]) {
+  constexpr int N = 2 * H;
+  z[0] = c32{p[0].x + p[0].y, p[0].x - p[0].y};
+  staticFor<H - 1>([&](auto kk) {
+    constexpr int k = decltype(kk)::value + 1;
+    c32 a = p[k];
+    c32 b = p[H - k];
+    // E2 = a + conj b, O2 = (a - conj b) W_N^{-k}, Z = E2 + i O2
+    c32 e = c32{a.x + b.x, a.y - b.y};
+    c32 d = c32{a.x - b.x, a.y + b.y};
+    c32 o = mulRoot<N, k, false>(d);
+    z[k] = c32{e.x - o.y, e.y + o.x};
+  });
+}
+
+}  // namespace fbfft_amd

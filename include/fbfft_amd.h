@@ -1,0 +1,156 @@
+/*
+ * fbfft_amd.h - C ABI of the MI355X (gfx950) implementation of fbcuda's fbfft path.
+ *
+ * Every entry point takes plain pointers, sizes and strides; no C++ or torch
+ * types cross this boundary.  All work is enqueued on the caller's HIP stream
+ * and nothing is synchronised.  Buffers (including scratch for the two-call
+ * 64/128 forms and the device arrays of tile descriptors) are owned by the
+ * caller.  The library keeps no mutable global state.
+ *
+ * File:line citations name the reference interface each declaration replaces
+ * (paths relative to the fbcuda source tree).
+ */
+#ifndef FBFFT_AMD_H
+#define FBFFT_AMD_H
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* hipStream_t is "struct ihipStream_t*"; declared here so that C callers do not
+ * need the HIP headers. */
+struct ihipStream_t;
+typedef struct ihipStream_t* fbfft_stream_t;
+
+/* FBFFTParameters::ErrorCode (fbfft/FBFFTParameters.h:9-14).  HipError takes the
+ * place of CudaError.  Invariant violations that abort in the reference (glog
+ * CHECK / assert) are reported as UnsupportedDimension or UnsupportedSize. */
+enum fbfft_error {
+  FBFFT_SUCCESS = 0,
+  FBFFT_UNSUPPORTED_SIZE = 1,
+  FBFFT_UNSUPPORTED_DIMENSION = 2,
+  FBFFT_HIP_ERROR = 3
+};
+
+/* A non-owning strided view: the contents of DeviceTensor<float, dim>
+ * (DeviceTensor.cuh:237-245: data pointer, then strides, then sizes), strides
+ * in units of float.  Complex tensors are float tensors whose innermost
+ * dimension has size 2 and stride 1. */
+#define FBFFT_MAX_DIM 5
+typedef struct fbfft_tensor {
+  float* data;
+  int stride[FBFFT_MAX_DIM];
+  int size[FBFFT_MAX_DIM];
+  int dim;
+} fbfft_tensor;
+
+/* TiledDeviceTensor<float, 4> (fbfft/FFTIteratedConvolution.cuh:71-88): 48 bytes,
+ * layout-compatible with the reference so existing host code that builds and
+ * uploads the descriptor arrays keeps working. */
+typedef struct fbfft_tile {
+  int padL;
+  int padU;
+  float* data;
+  int stride[4];
+  int size[4];
+} fbfft_tile;
+
+/* FFTConvolutionPassFFI (fbfft/FFTIteratedConvolution.cuh:616-622) */
+enum fbfft_conv_pass {
+  FBFFT_UPDATE_OUTPUT = 0,
+  FBFFT_UPDATE_GRAD_INPUT = 1,
+  FBFFT_ACC_GRAD_PARAMETERS = 2
+};
+
+/* fbfft1D<1> (fbfft/FBFFT.cuh:11-16, fbfft/FBFFT-inl.cuh:19-87).
+ * real [B][N] -> cplx [B][N/2+1][2], N = real->size[1], a power of two in
+ * [2, 256].  padL shifts the row right and drops its last padL samples. */
+int fbfft_r2c_1d(const fbfft_tensor* real, const fbfft_tensor* cplx, int padL,
+                 fbfft_stream_t stream);
+
+/* fbifft1D<1> (fbfft/FBFFT.cuh:18-23, fbfft/FBFFT-inl.cuh:89-150).
+ * cplx [B][N/2+1][2] -> real [B][N], unnormalised (gain N). */
+int fbfft_c2r_1d(const fbfft_tensor* real, const fbfft_tensor* cplx, int padL,
+                 fbfft_stream_t stream);
+
+/* fbfft2D<1>(real, complexAsFloat, padL, padU) (fbfft/FBFFT.cuh:30-36,
+ * fbfft/FBFFT2D-inl.cuh:450-623).
+ * real [B][h][w] is placed at (padU, padL) of a zero N x N plane.
+ *   cplx [B][N/2+1][N][2], N in {8,16,32}:  cplx[b][ky][kx]  (one kernel)
+ *   cplx [B][N/2+1][N][2], N in {64,128}:   cplx[b][kx][ky]  (one kernel; an
+ *       extension: the reference needs two calls and a scratch buffer)
+ *   cplx [B][N][N/2+1][2], N in {64,128}:   the reference's first pass: row
+ *       transforms into the caller's scratch, cplx[b][y][kx]. */
+int fbfft_r2c_2d(const fbfft_tensor* real, const fbfft_tensor* cplx, int padL, int padU,
+                 fbfft_stream_t stream);
+
+/* fbfft2D<1>(Complex src, Complex dst) (fbfft/FBFFT.cuh:39-43,
+ * fbfft/FBFFT2D-inl.cuh:627-669): second pass for N in {64,128}.
+ * src [B][N][N/2+1][2] (scratch) -> dst [B][N/2+1][N][2], dst[b][kx][ky]. */
+int fbfft_c2c_2d_pass2(const fbfft_tensor* src, const fbfft_tensor* dst, fbfft_stream_t stream);
+
+/* fbifft2D<1>(Complex src, real dst, padL, padU) (fbfft/FBFFT.cuh:50-56,
+ * fbfft/FBIFFT2D-inl.cuh:567-742).  Unnormalised (gain N*N); only the window of
+ * the N x N result that real covers at (padU, padL) is written.
+ *   cplx [B][N/2+1][N][2], N in {8,16,32}:  one kernel
+ *   cplx [B][N/2+1][N][2], N in {64,128}:   one kernel (extension, as above)
+ *   cplx [B][N][N][2],     N in {64,128}:   the reference's second inverse pass
+ *       over the scratch produced by fbfft_c2c_2d_inverse_pass1. */
+int fbfft_c2r_2d(const fbfft_tensor* cplx, const fbfft_tensor* real, int padL, int padU,
+                 fbfft_stream_t stream);
+
+/* fbifft2D<1>(float src, float dst) (fbfft/FBFFT.cuh:45-49,
+ * fbfft/FBIFFT2D-inl.cuh:529-563): first inverse pass for N in {64,128}.
+ * src [B][N/2+1][N][2] -> dst [B][N][N][2] scratch; planes b and b + ceil(B/2)
+ * share one complex transform, so only the first ceil(B/2) planes of dst are
+ * written. */
+int fbfft_c2c_2d_inverse_pass1(const fbfft_tensor* src, const fbfft_tensor* dst,
+                               fbfft_stream_t stream);
+
+/* transposeMM<Dim, ConjugateTransposeA, ConjugateTransposeB, Accumulate>
+ * (MM.cuh:11-17, MM-inl.cuh:515-814).  Operands are float tensors of rank 3..5
+ * whose last dimension is the (re, im) pair and whose dimensions between the
+ * first two and the last are contiguous and collapse to xy:
+ *   A [I][K][xy][2] (conjA: [K][I][xy][2]),  B [K][J][xy][2] (conjB: [J][K][xy][2])
+ *   C[i][j][xy] = invNorm * ((accumulate ? C[i][j][xy] : 0) + sum_k opA * opB)
+ * where opX conjugates when conjX is set.  Returns an fbfft_error (the
+ * reference returns void and aborts on bad shapes). */
+int fbfft_transpose_mm(const fbfft_tensor* A, const fbfft_tensor* B, const fbfft_tensor* C,
+                       int conjA, int conjB, int accumulate, float invNorm,
+                       fbfft_stream_t stream);
+
+/* detail::FFTIteratedConvolution<FFTSize> (fbfft/FFTIteratedConvolution.cuh:624-755).
+ * ins / outs are DEVICE pointers to numTiles descriptors each.  weight is
+ * [Cout][Cin][kH][kW].  Returns 1 if a kernel was launched, 0 if the pass code or
+ * FFT size matched nothing (the reference's bool), and a negative fbfft_error
+ * (-FBFFT_HIP_ERROR ...) on launch failure. */
+int fbfft_iterated_conv(int fftSize, const fbfft_tile* ins, const fbfft_tile* outs,
+                        const fbfft_tensor* weight, int pass, float scale, int batchSize,
+                        size_t numTiles, fbfft_stream_t stream);
+
+/* Bytes of device workspace fbfft_conv_fprop needs for the given problem. */
+size_t fbfft_conv_fprop_workspace(int batch, int cin, int cout, int fftSize);
+
+/* FFT convolution forward pass: the FFT -> transposeMM<false,true> -> IFFT
+ * sequence that the reference's external callers compose from the primitives
+ * above (MM-inl.cuh:188-196 role table).  Valid cross-correlation (no kernel
+ * flip): input [B][Cin][H][W], weight [Cout][Cin][kH][kW], H, W <= fftSize in
+ * {8,16,32}, output [B][Cout][H-kH+1][W-kW+1].  workspace: device memory of at
+ * least fbfft_conv_fprop_workspace() bytes, 256-byte aligned. */
+int fbfft_conv_fprop(const fbfft_tensor* input, const fbfft_tensor* weight,
+                     const fbfft_tensor* output, int fftSize, void* workspace,
+                     size_t workspaceBytes, fbfft_stream_t stream);
+
+/* Human-readable name of an fbfft_error. */
+const char* fbfft_error_string(int code);
+
+/* The 128-entry (cos, sin)(k*pi/128) table the kernels are built with
+ * (fbfft/Twiddles.cuh:322-453); copies 256 floats to out. */
+void fbfft_twiddle_table(float* out);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FBFFT_AMD_H */

@@ -1,0 +1,41 @@
+"""Shared helpers of the GPU parity tests: they call the product through its C ABI
+(fbcuda_amd -> libfbfft_amd.so) and check it against the CPU oracle."""
+import numpy as np
+import torch
+
+import fbcuda_amd as F
+
+TOL_FFT = 1e-5    # rel-L2 per transform (vs the fp32 transcription and vs the fp64 DFT)
+TOL_CONV = 1e-4   # rel-L2 per full convolution
+
+
+def dev():
+    return torch.device("cuda:0")
+
+
+def c(a):
+    a = np.asarray(a)
+    return a[..., 0] + 1j * a[..., 1]
+
+
+def rel(a, b):
+    a = np.asarray(a, dtype=np.float64).ravel()
+    b = np.asarray(b, dtype=np.float64).ravel()
+    return float(np.linalg.norm(a - b) / max(np.linalg.norm(b), 1e-300))
+
+
+def fft2d(x, N, padL=0, padU=0):
+    """numpy real [B][h][w] -> numpy [B][N/2+1][N][2] through the C ABI."""
+    xd = torch.from_numpy(np.ascontiguousarray(x, dtype=np.float32)).to(dev())
+    out = torch.full((x.shape[0], N // 2 + 1, N, 2), float("nan"), device=dev())
+    rc = F.fbfft2D(xd, out, padL, padU)
+    torch.cuda.synchronize()
+    return rc, out.cpu().numpy()
+
+
+def ifft2d(spec, h, w, padL=0, padU=0, fill=float("nan")):
+    sd = torch.from_numpy(np.ascontiguousarray(spec, dtype=np.float32)).to(dev())
+    out = torch.full((spec.shape[0], h, w), fill, device=dev())
+    rc = F.fbifft2D(sd, out, padL, padU)
+    torch.cuda.synchronize()
+    return rc, out.cpu().numpy()

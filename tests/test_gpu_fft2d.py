@@ -1,0 +1,135 @@
+"""GPU parity of fbfft2D / fbifft2D (C ABI fbfft_r2c_2d / fbfft_c2r_2d) against
+the CPU oracle: fp32 transcription, fp64 DFT, golden fixtures, edge cases and
+size-independent properties at the benchmark's full size."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import fbcuda_amd as F
+from fbcuda_amd import synth
+from gpu_util import TOL_FFT, c, dev, fft2d, ifft2d, rel
+
+pytestmark = pytest.mark.gpu
+GOLD = np.load(os.path.join(os.path.dirname(__file__), "golden", "fft_vectors.npz"))
+SIZES = [8, 16, 32, 64, 128]
+
+
+@pytest.mark.parametrize("key", [k[4:] for k in GOLD.files if k.startswith("x2d_")])
+def test_golden(key):
+    N, h, w, padL, padU = map(int, key.split("_"))
+    rc, out = fft2d(GOLD["x2d_" + key], N, padL, padU)
+    assert rc == F.Success
+    assert rel(c(out), GOLD["f2d_" + key]) < TOL_FFT
+
+
+@pytest.mark.parametrize("N", SIZES)
+@pytest.mark.parametrize("case", ["full", "ragged", "padded", "tiny"])
+@pytest.mark.parametrize("B", [1, 5, 67])
+def test_forward_inverse_vs_oracle(oracle, N, case, B):
+    h, w, padL, padU = {"full": (N, N, 0, 0), "ragged": (N - 5, N - 3, 0, 0),
+                        "padded": (N - 5, N - 4, 2, 3), "tiny": (5, 5, 0, 0)}[case]
+    x = synth.normal((B, h, w), seed=N + B).numpy()
+    rc, got = fft2d(x, N, padL, padU)
+    assert rc == F.Success
+    _, want32 = oracle.fbfft2d(x, N, padL, padU)
+    want64 = oracle.dft2d_r2c(x, N, padL, padU)
+    assert rel(got, want32) < TOL_FFT
+    assert rel(got, want64) < TOL_FFT
+    # inverse of the oracle's spectrum, cropped on store; cells outside stay untouched
+    rc, back = ifft2d(want32, h, w, padL, padU)
+    assert rc == F.Success
+    _, back32 = oracle.fbifft2d(want32, h, w, padL, padU)
+    assert rel(back, back32) < TOL_FFT
+    assert rel(back, N * N * x.astype(np.float64)) < TOL_FFT
+
+
+@pytest.mark.parametrize("N", SIZES)
+def test_inverse_writes_only_the_window(oracle, N):
+    """crop-on-store: a real tensor smaller than N x N receives exactly its window."""
+    x = synth.normal((3, N, N), seed=77).numpy()
+    _, spec = oracle.fbfft2d(x, N)
+    h, w, padL, padU = N - 9 if N > 9 else 3, N - 5, 1, 2
+    rc, got = ifft2d(spec, h, w, padL, padU)
+    assert rc == F.Success
+    want = N * N * x[:, padU:padU + h, padL:padL + w].astype(np.float64)
+    assert rel(got, want) < TOL_FFT
+
+
+@pytest.mark.parametrize("N", [8, 16, 32])
+def test_inverse_lane0_quirk(oracle, N):
+    """Imaginary parts of F[0][0] and F[N/2][0] are ignored (fbfft/FFT2D32.cuh:313-315)."""
+    x = synth.normal((2, N, N), seed=5).numpy()
+    _, spec = oracle.fbfft2d(x, N)
+    spec[:, 0, 0, 1] = 3.0
+    spec[:, N // 2, 0, 1] = -4.0
+    _, got = ifft2d(spec, N, N)
+    _, want = oracle.fbifft2d(spec, N, N)
+    assert rel(got, want) < TOL_FFT
+    assert rel(got, N * N * x.astype(np.float64)) < TOL_FFT
+
+
+@pytest.mark.parametrize("N", SIZES)
+def test_strided_operands(oracle, N):
+    """Non-contiguous views: padded batch / row strides on both operands."""
+    B = 6
+    x = synth.normal((B, N, N), seed=9).numpy()
+    big = torch.zeros((B, N + 3, N + 4), device=dev())
+    real = big[:, 1:N + 1, 2:N + 2]
+    real.copy_(torch.from_numpy(x))
+    wide = torch.full((B, N // 2 + 2, N + 2, 2), float("nan"), device=dev())
+    spec = wide[:, :N // 2 + 1, 1:N + 1, :]
+    assert F.fbfft2D(real, spec) == F.Success
+    torch.cuda.synchronize()
+    _, want = oracle.fbfft2d(x, N)
+    assert rel(spec.cpu().numpy(), want) < TOL_FFT
+    back = torch.zeros_like(big)
+    assert F.fbifft2D(spec, back[:, 1:N + 1, 2:N + 2]) == F.Success
+    torch.cuda.synchronize()
+    assert rel(back[:, 1:N + 1, 2:N + 2].cpu().numpy(), N * N * x.astype(np.float64)) < TOL_FFT
+    assert float(back[:, 0].abs().max()) == 0.0  # nothing outside the view was written
+
+
+def test_error_codes():
+    d = dev()
+    real = torch.zeros((4, 32, 32), device=d)
+    assert F.fbfft2D(real, torch.zeros((4, 17, 32, 2), device=d)) == F.Success
+    assert F.fbfft2D(real, torch.zeros((4, 129, 256, 2), device=d)) == F.UnsupportedSize
+    assert F.fbfft2D(real, torch.zeros((4, 7, 12, 2), device=d)) == F.UnsupportedSize
+    assert F.fbfft2D(real, torch.zeros((4, 16, 32, 2), device=d)) == F.UnsupportedSize
+    assert F.fbfft2D(real, torch.zeros((3, 17, 32, 2), device=d)) == F.UnsupportedDimension
+    assert F.fbfft2D(real, torch.zeros((4, 17, 32), device=d)) == F.UnsupportedDimension
+    assert F.fbfft2D(torch.zeros((4, 40, 32), device=d),
+                     torch.zeros((4, 17, 32, 2), device=d)) == F.UnsupportedSize
+    assert F.fbifft2D(torch.zeros((4, 129, 256, 2), device=d), real) == F.UnsupportedSize
+    # empty batch is a successful no-op
+    assert F.fbfft2D(torch.zeros((0, 32, 32), device=d), torch.zeros((0, 17, 32, 2), device=d)) == F.Success
+    torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("N,B", [(32, 16384), (8, 1 << 20), (16, 1 << 18), (64, 16384), (128, 4096)])
+def test_full_size_properties(oracle, N, B):
+    """Benchmark sizes: round trip ifft(fft(x)) = N^2 x on the whole tensor,
+    linearity, and oracle parity on a seeded subset of planes."""
+    d = dev()
+    seed = {32: 1, 8: 5, 16: 6, 64: 8, 128: 9}[N]
+    x = synth.normal((B, N, N), seed=seed, device=d)
+    spec = torch.empty((B, N // 2 + 1, N, 2), device=d)
+    assert F.fbfft2D(x, spec) == F.Success
+    back = torch.empty_like(x)
+    assert F.fbifft2D(spec, back) == F.Success
+    torch.cuda.synchronize()
+    err = (back / (N * N) - x).double().norm() / x.double().norm()
+    assert float(err) < TOL_FFT
+    pick = [0, 1, B // 3, B // 2 + 1, B - 2, B - 1]
+    _, want = oracle.fbfft2d(x[pick].cpu().numpy(), N)
+    assert rel(spec[pick].cpu().numpy(), want) < TOL_FFT
+    # linearity on a slice: F(2x + y) = 2F(x) + F(y)
+    n = min(B // 2, 4096)
+    z = (2 * x[:n] + x[n:2 * n]).contiguous()
+    sz = torch.empty((n, N // 2 + 1, N, 2), device=d)
+    assert F.fbfft2D(z, sz) == F.Success
+    torch.cuda.synchronize()
+    lin = (sz - (2 * spec[:n] + spec[n:2 * n])).double().norm() / sz.double().norm()
+    assert float(lin) < TOL_FFT
