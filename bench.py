@@ -1,0 +1,193 @@
+#!/usr/bin/env python3
+"""Benchmark of the fbfft hot path on one MI355X.
+
+A step is one fbfft2D real-to-complex pass over the whole batch of
+BASELINE.json configs[1] (16384 planes of 32x32 fp32, N(0,1), seed 1), inputs
+resident in HBM.  Prints ONE JSON line:
+
+  value / unit   algorithmic GB/s of the timed region (8448 bytes per plane:
+                 4096 read + 4352 written), the metric BASELINE.json names
+  roofline       the R2C kernel against the 8 TB/s HBM peak, duration from HIP
+                 events recorded on the launch stream around the timed region
+  cpu_baseline   the CPU oracle (host transcription of the reference's
+                 algorithm, OpenMP over planes) on the same workload, timed on
+                 this machine's cores for a bounded number of passes
+  extra          other measured configurations (C2R, other sizes, the FFT
+                 convolution of configs[3]) - informative, not the metric
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+
+
+def plane_bytes(N):
+    return 4 * N * N + 8 * N * (N // 2 + 1)
+
+
+def timed(fn, steps, warmup, torch):
+    """(seconds per step by host clock with sync on both sides, seconds per launch by HIP events)."""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    e0 = torch.cuda.Event(enable_timing=True)
+    e1 = torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(steps):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    return (t1 - t0) / steps, e0.elapsed_time(e1) * 1e-3 / steps
+
+
+def prepared(fn_name, F, *tensors_then_ints):
+    """Bind a C-ABI call once: descriptors are built outside the timed region."""
+    import torch
+    L = F.lib()
+    cfn = getattr(L, fn_name)
+    args = []
+    keep = []
+    for a in tensors_then_ints:
+        if isinstance(a, torch.Tensor):
+            v = F.view(a)
+            keep.append(v)
+            args.append(ctypes.byref(v))
+        else:
+            args.append(a)
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    args.append(stream)
+
+    def call():
+        rc = cfn(*args)
+        if rc != 0:
+            raise RuntimeError("%s failed: %s" % (fn_name, F.error_string(rc)))
+    call.keep = keep
+    return call
+
+
+def cpu_baseline(x_host, N, budget_s=12.0):
+    """Times the CPU oracle (kind "port") on the same planes; bounded to ~budget_s."""
+    import oracle as O
+    threads = O.num_threads()
+    O.fbfft2d(x_host[:64], N)  # warm
+    t0 = time.perf_counter()
+    O.fbfft2d(x_host, N)
+    one = time.perf_counter() - t0
+    reps = max(1, min(50, int(budget_s / max(one, 1e-3))))
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        O.fbfft2d(x_host, N)
+    dt = (time.perf_counter() - t0) / reps
+    gbs = x_host.shape[0] * plane_bytes(N) / dt / 1e9
+    return {"value": round(gbs, 3), "unit": "GB/s", "cores": threads, "kind": "port",
+            "sample": "%d passes of the full %d-plane %dx%d R2C batch, OpenMP over planes, "
+                      "%.3f s per pass" % (reps, x_host.shape[0], N, N, dt)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
+    ap.add_argument("--no-extra", action="store_true", help="skip the informative extra configs")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="only run a plain 256 MiB device-to-device copy 20 times: the known-size "
+                         "kernel that FETCH_SIZE / WRITE_SIZE counter readings are scaled by")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on exactly one GPU (no sharding or collectives "
+                 "are part of the fbfft path); run with --gpus 1")
+
+    import torch
+
+    import fbcuda_amd as F
+    from fbcuda_amd import synth
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible")
+    dev = torch.device("cuda:0")
+    F.lib()
+
+    if args.calibrate_copy:
+        a = torch.zeros(64 * 1024 * 1024, device=dev)
+        c = torch.empty_like(a)
+        for _ in range(20):
+            c.copy_(a)
+        torch.cuda.synchronize()
+        print(json.dumps({"calibrate_copy_bytes_read": a.numel() * 4,
+                          "calibrate_copy_bytes_written": a.numel() * 4, "launches": 20}))
+        return
+
+    N, B = 32, 16384
+    x = synth.normal((B, N, N), seed=1, device=dev)
+    spec = torch.empty((B, N // 2 + 1, N, 2), device=dev)
+    back = torch.empty_like(x)
+    fwd = prepared("fbfft_r2c_2d", F, x, spec, 0, 0)
+    inv = prepared("fbfft_c2r_2d", F, spec, back, 0, 0)
+
+    step_s, launch_s = timed(fwd, args.steps, args.warmup, torch)
+    nbytes = B * plane_bytes(N)
+    value = nbytes / step_s / 1e9
+    achieved = nbytes / launch_s / 1e9
+
+    extra = {}
+    if not args.no_extra:
+        s, l = timed(inv, args.steps, args.warmup, torch)
+        extra["c2r_32x32_b16384_GBps"] = round(nbytes / l / 1e9, 1)
+        # round-trip sanity on the benchmark tensors themselves
+        err = float((back / (N * N) - x).double().norm() / x.double().norm())
+        extra["roundtrip_rel_l2"] = err
+        for n2, b2 in ((32, 65536), (16, 262144), (8, 1048576), (64, 16384), (128, 4096)):
+            x2 = synth.normal((b2, n2, n2), seed=2 + n2.bit_length() - 1, device=dev)
+            s2 = torch.empty((b2, n2 // 2 + 1, n2, 2), device=dev)
+            f2 = prepared("fbfft_r2c_2d", F, x2, s2, 0, 0)
+            i2 = prepared("fbfft_c2r_2d", F, s2, x2, 0, 0)
+            try:
+                _, lf = timed(f2, 20, 5, torch)
+                _, li = timed(i2, 20, 5, torch)
+            except RuntimeError:
+                continue
+            nb = b2 * plane_bytes(n2)
+            extra["r2c_%dx%d_b%d_GBps" % (n2, n2, b2)] = round(nb / lf / 1e9, 1)
+            extra["c2r_%dx%d_b%d_GBps" % (n2, n2, b2)] = round(nb / li / 1e9, 1)
+            del x2, s2
+
+    out = {
+        "metric": "fbfft2D 32x32 R2C GB/s (% HBM peak); FFT-conv ms/iter at configs[3]",
+        "value": round(value, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(step_s * 1e3, 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": "configs[1]: fbfft2D R2C, 16384 planes of 32x32 fp32 N(0,1) seed 1, "
+                               "output [16384][17][32][2]; 8448 algorithmic bytes per plane"},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "kernel": "fft2dSmallForward<32>", "bytes_per_launch": nbytes,
+                     "launch_us": round(launch_s * 1e6, 2)},
+        "extra": extra,
+    }
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline(x.cpu().numpy(), N)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -82,7 +82,8 @@ int fbfft_r2c_2d(const fbfft_tensor* real, const fbfft_tensor* cplx, int padL, i
   if (!okCplx(cplx)) return FBFFT_UNSUPPORTED_DIMENSION;
   if (empty(real) || empty(cplx)) return FBFFT_SUCCESS;
   if (N <= 32) return launchFft2dSmallForward(N, realView3(real), cplxView4(cplx), padL, padU, stream);
-  (void)scratchForm;
+  if (!scratchForm)
+    return launchFft2dLargeForward(N, realView3(real), cplxView4(cplx), padL, padU, stream);
   return FBFFT_UNSUPPORTED_SIZE;
 }
 
@@ -100,6 +101,7 @@ int fbfft_c2r_2d(const fbfft_tensor* cplx, const fbfft_tensor* real, int padL, i
   if (!okCplx(cplx)) return FBFFT_UNSUPPORTED_DIMENSION;
   if (empty(real) || empty(cplx)) return FBFFT_SUCCESS;
   if (N <= 32) return launchFft2dSmallInverse(N, cplxView4(cplx), realView3(real), padL, padU, stream);
+  if (half) return launchFft2dLargeInverse(N, cplxView4(cplx), realView3(real), padL, padU, stream);
   return FBFFT_UNSUPPORTED_SIZE;
 }
 

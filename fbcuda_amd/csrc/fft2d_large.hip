@@ -1,0 +1,358 @@
+// 2D real-to-complex / complex-to-real transforms for N in {64, 128} in ONE
+// kernel and one pass over HBM.  The reference needs two kernels and a scratch
+// round trip for these sizes (fbfft/FBFFT2D-inl.cuh:230-444,
+// fbfft/FBIFFT2D-inl.cuh:252-521).  Output layout cplx[b][kx][ky], kx = 0..N/2:
+// the Hermitian-halved axis is the horizontal frequency and the plane is stored
+// transposed, as the reference's second pass leaves it.
+//
+// One workgroup owns one plane, which stays in LDS between the passes (one
+// buffer, reused by every stage):
+//   1. coalesced 16-byte loads of the real plane into LDS, rows padded by 4 floats;
+//   2. row pass: lane y turns row y (N reals) into N/2 packed complex values and
+//      runs an N/2-point complex FFT in VGPRs plus the real-input fix-up;
+//      columns kx = 0 and kx = N/2 (both real along y) travel packed as one;
+//   3. the result is written back transposed ([kx][y], odd row stride: no bank
+//      conflicts either way);
+//   4. column pass: each N-point column FFT is split over G lanes (G = 2 for 64,
+//      G = 4 for 128; for 128 G is the wave index): lane g forms the radix-G
+//      decimation-in-frequency sums for its residue straight from LDS, applies
+//      W_N^(g*j) from an LDS copy of the twiddle table and finishes with a
+//      32-point FFT in VGPRs;
+//   5. results return to LDS as [kx][ky] and leave as one contiguous stream of
+//      16-byte stores; the packed column is unpacked on the way out.
+// The inverse runs the same steps backwards and crops on store.
+#include "common.h"
+#include "fft_regs.h"
+
+namespace fbfft_amd {
+namespace {
+
+template <int N>
+struct LargeCfg {
+  static constexpr int H = N / 2;
+  static constexpr int G = (N == 64) ? 2 : 4;   // lanes per column FFT
+  static constexpr int L = N / G;               // points per lane in the column pass (32)
+  static constexpr int THREADS = H * G;         // 64 or 256
+  static constexpr int RSF = N + 4;             // real-plane row stride in floats
+  static constexpr int CS = N + 1;              // [kx][y|ky] row stride in complex
+  static constexpr int YS = H + 1;              // [y][kx] row stride in complex (inverse)
+  static constexpr int BUF_FLOATS =
+      (N * RSF > 2 * H * CS ? (N * RSF > 2 * N * YS ? N * RSF : 2 * N * YS)
+                            : (2 * H * CS > 2 * N * YS ? 2 * H * CS : 2 * N * YS));
+  static constexpr int F4_REAL = N * N / 4;           // float4 per real plane
+  static constexpr int F4_CPLX = (H + 1) * N / 2;     // float4 per spectrum plane
+};
+
+// full-circle twiddles e^{-/+ 2 pi i m / 256}, m = 0..255, from the half-circle table
+template <bool FWD, int THREADS>
+__device__ __forceinline__ void fillTwiddles(c32* tw, int t) {
+  for (int m = t; m < 256; m += THREADS) {
+    const int h = m & 127;
+    float c = __builtin_bit_cast(float, kTwiddleBits[2 * h]);
+    float s = __builtin_bit_cast(float, kTwiddleBits[2 * h + 1]);
+    if (m >= 128) {
+      c = -c;
+      s = -s;
+    }
+    tw[m] = c32{c, FWD ? -s : s};
+  }
+}
+
+// Lane g of G computes outputs X[G*k + g], k = 0..N/G-1, of the N-point FFT of
+// col[0..N) (LDS, unit stride); they are left in v[slot<N/G>(k)].
+template <int N, int G, bool FWD>
+__device__ __forceinline__ void splitColumnFFT(const c32* col, int g, const c32* tw,
+                                               c32 (&v)[N / G]) {
+  constexpr int L = N / G;
+  static_assert(G == 2 || G == 4, "column split");
+  if constexpr (G == 2) {
+    const float sgn = g ? -1.0f : 1.0f;
+    staticFor<L>([&](auto jj) {
+      constexpr int j = decltype(jj)::value;
+      c32 u0 = col[j], u1 = col[j + L];
+      c32 comb = c32{u0.x + sgn * u1.x, u0.y + sgn * u1.y};
+      c32 w = tw[(g * (j * (256 / N))) & 255];
+      v[j] = cmul(comb, w);
+    });
+  } else {
+    const float sA = (g & 1) ? -1.0f : 1.0f;
+    const bool rot = (g & 1) != 0;
+    // forward: omega = -i  -> g=1: -i*b, g=3: +i*b;  inverse: the other way round
+    const float sB = (g == 0) ? 1.0f : (g == 2) ? -1.0f : ((g == 1) == FWD) ? -1.0f : 1.0f;
+    staticFor<L>([&](auto jj) {
+      constexpr int j = decltype(jj)::value;
+      c32 u0 = col[j], u1 = col[j + L], u2 = col[j + 2 * L], u3 = col[j + 3 * L];
+      c32 a = c32{u0.x + sA * u2.x, u0.y + sA * u2.y};
+      c32 b = c32{u1.x + sA * u3.x, u1.y + sA * u3.y};
+      c32 br = rot ? c32{-b.y, b.x} : b;  // i*b when rot
+      c32 comb = c32{a.x + sB * br.x, a.y + sB * br.y};
+      c32 w = tw[(g * (j * (256 / N))) & 255];
+      v[j] = cmul(comb, w);
+    });
+  }
+  difFFT<L, FWD>(v);
+}
+
+template <int N, bool FAST_REAL, bool FAST_CPLX>
+__global__ __launch_bounds__(LargeCfg<N>::THREADS) void fft2dLargeForward(RealView real,
+                                                                         CplxView cplx, int padL,
+                                                                         int padU) {
+  using C = LargeCfg<N>;
+  constexpr int H = C::H, G = C::G, L = C::L, THREADS = C::THREADS, RSF = C::RSF, CS = C::CS;
+  __shared__ __align__(16) float buf[C::BUF_FLOATS];
+  __shared__ __align__(8) c32 tw[256];
+  const int t = threadIdx.x;
+  const int b = blockIdx.x;
+  fillTwiddles<true, THREADS>(tw, t);
+
+  // ---- 1. real plane -> LDS [y][x] ----
+  if constexpr (FAST_REAL) {
+    const float4* src = reinterpret_cast<const float4*>(real.data + (size_t)b * real.sb);
+    const int rs4 = real.sy / 4;
+    staticFor<C::F4_REAL / THREADS>([&](auto ii) {
+      constexpr int i = decltype(ii)::value;
+      const int q = t + THREADS * i;
+      const int y = q / (N / 4), x4 = q % (N / 4);
+      *reinterpret_cast<float4*>(buf + y * RSF + 4 * x4) = src[(size_t)y * rs4 + x4];
+    });
+  } else {
+    const float* src = real.data + (size_t)b * real.sb;
+    for (int q = t; q < N * N; q += THREADS) {
+      const int y = q / N, x = q % N;
+      buf[y * RSF + x] = inWindow(y, x, padU, padL, real.h, real.w)
+                             ? src[(size_t)(y - padU) * real.sy + (size_t)(x - padL) * real.sx]
+                             : 0.0f;
+    }
+  }
+  __syncthreads();
+
+  // ---- 2. row pass: lane y, N reals -> H packed complex ----
+  c32 z[H];
+  if (t < N) {
+    const float* row = buf + t * RSF;
+    staticFor<H / 2>([&](auto mm) {
+      constexpr int m = decltype(mm)::value;
+      float4 v = *reinterpret_cast<const float4*>(row + 4 * m);
+      z[2 * m] = c32{v.x, v.y};
+      z[2 * m + 1] = c32{v.z, v.w};
+    });
+  }
+  __syncthreads();  // every row is in registers: the buffer may be overwritten
+  c32* cb = reinterpret_cast<c32*>(buf);
+  if (t < N) {
+    difFFT<H, true>(z);
+    // ---- 3. fix-up fused with the transposed write: [kx][y] ----
+    realFixupForwardEmit<H>(z, [&](auto kk, c32 val) {
+      constexpr int k = decltype(kk)::value;
+      cb[k * CS + t] = val;
+    });
+  }
+  __syncthreads();
+
+  // ---- 4. column pass ----
+  const int col = t % H, g = t / H;
+  c32 v[L];
+  splitColumnFFT<N, G, true>(cb + col * CS, g, tw, v);
+  __syncthreads();  // all columns consumed
+  // ---- 5. [kx][ky] back to LDS ----
+  staticFor<L>([&](auto kk) {
+    constexpr int k = decltype(kk)::value;
+    cb[col * CS + G * k + g] = v[slot<L>(k)];
+  });
+  __syncthreads();
+
+  // ---- copy out (H+1) x N complex; rows 0 and H come from packed row 0 ----
+  constexpr int ITERS = (C::F4_CPLX + THREADS - 1) / THREADS;
+  staticFor<ITERS>([&](auto ii) {
+    constexpr int i = decltype(ii)::value;
+    const int q = t + THREADS * i;
+    if (q < C::F4_CPLX) {
+      const int r = q / (N / 2);
+      const int ky = 2 * (q % (N / 2));
+      float4 o;
+      if (r == 0 || r == H) {
+        c32 a0 = cb[ky], a1 = cb[ky + 1];
+        c32 m0 = cb[(N - ky) & (N - 1)], m1 = cb[N - ky - 1];
+        if (r == 0)
+          o = float4{0.5f * (a0.x + m0.x), 0.5f * (a0.y - m0.y), 0.5f * (a1.x + m1.x),
+                     0.5f * (a1.y - m1.y)};
+        else
+          o = float4{0.5f * (a0.y + m0.y), 0.5f * (m0.x - a0.x), 0.5f * (a1.y + m1.y),
+                     0.5f * (m1.x - a1.x)};
+      } else {
+        c32 a0 = cb[r * CS + ky], a1 = cb[r * CS + ky + 1];
+        o = float4{a0.x, a0.y, a1.x, a1.y};
+      }
+      if constexpr (FAST_CPLX) {
+        reinterpret_cast<float4*>(cplx.data + (size_t)b * cplx.sb)[q] = o;
+      } else {
+        float* dst = cplx.data + (size_t)b * cplx.sb + (size_t)r * cplx.sr + (size_t)ky * cplx.sc;
+        *reinterpret_cast<float2*>(dst) = float2{o.x, o.y};
+        *reinterpret_cast<float2*>(dst + cplx.sc) = float2{o.z, o.w};
+      }
+    }
+  });
+}
+
+template <int N, bool FAST_REAL, bool FAST_CPLX>
+__global__ __launch_bounds__(LargeCfg<N>::THREADS) void fft2dLargeInverse(CplxView cplx,
+                                                                         RealView real, int padL,
+                                                                         int padU) {
+  using C = LargeCfg<N>;
+  constexpr int H = C::H, G = C::G, L = C::L, THREADS = C::THREADS, RSF = C::RSF, CS = C::CS,
+                YS = C::YS;
+  __shared__ __align__(16) float buf[C::BUF_FLOATS];
+  __shared__ __align__(8) c32 tw[256];
+  const int t = threadIdx.x;
+  const int b = blockIdx.x;
+  fillTwiddles<false, THREADS>(tw, t);
+  c32* cb = reinterpret_cast<c32*>(buf);
+
+  // ---- copy in [kx][ky]; row H is folded into row 0: Z = F0 + i*FH ----
+  constexpr int ITERS = (C::F4_CPLX + THREADS - 1) / THREADS;
+  // rows 0..H-1 first, then row H is added into row 0 after a barrier
+  staticFor<ITERS>([&](auto ii) {
+    constexpr int i = decltype(ii)::value;
+    const int q = t + THREADS * i;
+    if (q < H * (N / 2)) {
+      const int r = q / (N / 2);
+      const int ky = 2 * (q % (N / 2));
+      float4 v;
+      if constexpr (FAST_CPLX) {
+        v = reinterpret_cast<const float4*>(cplx.data + (size_t)b * cplx.sb)[q];
+      } else {
+        const float* src = cplx.data + (size_t)b * cplx.sb + (size_t)r * cplx.sr + (size_t)ky * cplx.sc;
+        float2 a = *reinterpret_cast<const float2*>(src);
+        float2 c = *reinterpret_cast<const float2*>(src + cplx.sc);
+        v = float4{a.x, a.y, c.x, c.y};
+      }
+      cb[r * CS + ky] = c32{v.x, v.y};
+      cb[r * CS + ky + 1] = c32{v.z, v.w};
+    }
+  });
+  __syncthreads();
+  if (t < N / 2) {
+    const int ky = 2 * t;
+    float4 v;
+    if constexpr (FAST_CPLX) {
+      v = reinterpret_cast<const float4*>(cplx.data + (size_t)b * cplx.sb)[H * (N / 2) + t];
+    } else {
+      const float* src = cplx.data + (size_t)b * cplx.sb + (size_t)H * cplx.sr + (size_t)ky * cplx.sc;
+      float2 a = *reinterpret_cast<const float2*>(src);
+      float2 c = *reinterpret_cast<const float2*>(src + cplx.sc);
+      v = float4{a.x, a.y, c.x, c.y};
+    }
+    c32 a0 = cb[ky], a1 = cb[ky + 1];
+    cb[ky] = c32{a0.x - v.y, a0.y + v.x};
+    cb[ky + 1] = c32{a1.x - v.w, a1.y + v.z};
+  }
+  __syncthreads();
+
+  // ---- column pass (inverse) ----
+  const int col = t % H, g = t / H;
+  c32 v[L];
+  splitColumnFFT<N, G, false>(cb + col * CS, g, tw, v);
+  __syncthreads();
+  // [y][kx]
+  staticFor<L>([&](auto kk) {
+    constexpr int k = decltype(kk)::value;
+    cb[(G * k + g) * YS + col] = v[slot<L>(k)];
+  });
+  __syncthreads();
+
+  // ---- row pass (inverse): lane y ----
+  c32 z[H];
+  if (t < N) {
+    const c32* row = cb + t * YS;
+    realFixupInverseFetch<H>([&](auto kk) { return row[decltype(kk)::value]; }, z);
+    difFFT<H, false>(z);
+  }
+  __syncthreads();
+  if (t < N) {
+    float* row = buf + t * RSF;
+    staticFor<H / 2>([&](auto mm) {
+      constexpr int m = decltype(mm)::value;
+      c32 a = z[slot<H>(2 * m)], c = z[slot<H>(2 * m + 1)];
+      *reinterpret_cast<float4*>(row + 4 * m) = float4{a.x, a.y, c.x, c.y};
+    });
+  }
+  __syncthreads();
+
+  // ---- copy out, cropped to the window real covers ----
+  if constexpr (FAST_REAL) {
+    float4* dst = reinterpret_cast<float4*>(real.data + (size_t)b * real.sb);
+    const int rs4 = real.sy / 4;
+    staticFor<C::F4_REAL / THREADS>([&](auto ii) {
+      constexpr int i = decltype(ii)::value;
+      const int q = t + THREADS * i;
+      const int y = q / (N / 4), x4 = q % (N / 4);
+      dst[(size_t)y * rs4 + x4] = *reinterpret_cast<const float4*>(buf + y * RSF + 4 * x4);
+    });
+  } else {
+    float* dst = real.data + (size_t)b * real.sb;
+    for (int q = t; q < N * N; q += THREADS) {
+      const int y = q / N, x = q % N;
+      if (inWindow(y, x, padU, padL, real.h, real.w))
+        dst[(size_t)(y - padU) * real.sy + (size_t)(x - padL) * real.sx] = buf[y * RSF + x];
+    }
+  }
+}
+
+bool fastReal(int N, const RealView& r, int padL, int padU) {
+  return padL == 0 && padU == 0 && r.h == N && r.w == N && r.sx == 1 && r.sy % 4 == 0 &&
+         r.sb % 4 == 0 && aligned(r.data, 16);
+}
+
+bool fastCplx(int N, const CplxView& c) {
+  return c.sc == 2 && c.sr == 2 * N && c.sb % 4 == 0 && aligned(c.data, 16);
+}
+
+template <int N>
+int launchForward(const RealView& real, const CplxView& cplx, int padL, int padU, hipStream_t s) {
+  dim3 grid(real.B), block(LargeCfg<N>::THREADS);
+  const bool fr = fastReal(N, real, padL, padU), fc = fastCplx(N, cplx);
+  if (fr && fc)
+    fft2dLargeForward<N, true, true><<<grid, block, 0, s>>>(real, cplx, padL, padU);
+  else if (fc)
+    fft2dLargeForward<N, false, true><<<grid, block, 0, s>>>(real, cplx, padL, padU);
+  else if (fr)
+    fft2dLargeForward<N, true, false><<<grid, block, 0, s>>>(real, cplx, padL, padU);
+  else
+    fft2dLargeForward<N, false, false><<<grid, block, 0, s>>>(real, cplx, padL, padU);
+  return launchStatus();
+}
+
+template <int N>
+int launchInverse(const CplxView& cplx, const RealView& real, int padL, int padU, hipStream_t s) {
+  dim3 grid(real.B), block(LargeCfg<N>::THREADS);
+  const bool fr = fastReal(N, real, padL, padU), fc = fastCplx(N, cplx);
+  if (fr && fc)
+    fft2dLargeInverse<N, true, true><<<grid, block, 0, s>>>(cplx, real, padL, padU);
+  else if (fc)
+    fft2dLargeInverse<N, false, true><<<grid, block, 0, s>>>(cplx, real, padL, padU);
+  else if (fr)
+    fft2dLargeInverse<N, true, false><<<grid, block, 0, s>>>(cplx, real, padL, padU);
+  else
+    fft2dLargeInverse<N, false, false><<<grid, block, 0, s>>>(cplx, real, padL, padU);
+  return launchStatus();
+}
+
+}  // namespace
+
+int launchFft2dLargeForward(int N, const RealView& real, const CplxView& cplx, int padL, int padU,
+                            hipStream_t s) {
+  if (real.B <= 0) return FBFFT_SUCCESS;
+  if (N == 64) return launchForward<64>(real, cplx, padL, padU, s);
+  if (N == 128) return launchForward<128>(real, cplx, padL, padU, s);
+  return FBFFT_UNSUPPORTED_SIZE;
+}
+
+int launchFft2dLargeInverse(int N, const CplxView& cplx, const RealView& real, int padL, int padU,
+                            hipStream_t s) {
+  if (real.B <= 0) return FBFFT_SUCCESS;
+  if (N == 64) return launchInverse<64>(cplx, real, padL, padU, s);
+  if (N == 128) return launchInverse<128>(cplx, real, padL, padU, s);
+  return FBFFT_UNSUPPORTED_SIZE;
+}
+
+}  // namespace fbfft_amd

@@ -103,45 +103,72 @@ constexpr int slot(int k) {
 }
 
 // Forward real-input fix-up.  z (in difFFT output order) is the H-point complex
-// FFT of z[j] = x[2j] + i*x[2j+1]; on return p[k], k = 1..H-1, holds F[k] of the
-// 2H-point real transform (natural order) and p[0] = (F[0], F[H]) packed as
-// (re, im) - both are real.
-template <int H>
-__device__ __forceinline__ void realFixupForward(const c32 (&z)[H], c32 (&p)[H]) {
+// FFT of z[j] = x[2j] + i*x[2j+1].  emit(k, value) is called once for every
+// k = 0..H-1 (k as an integral_constant) with F[k] of the 2H-point real
+// transform; for k = 0 the value is (F[0], F[H]) packed as (re, im) - both are
+// real.  Bins k and H-k share one twiddle product.
+template <int H, typename Emit>
+__device__ __forceinline__ void realFixupForwardEmit(const c32 (&z)[H], Emit&& emit) {
   constexpr int N = 2 * H;
   {
     c32 z0 = z[0];
-    p[0] = c32{z0.x + z0.y, z0.x - z0.y};
+    emit(std::integral_constant<int, 0>{}, c32{z0.x + z0.y, z0.x - z0.y});
   }
-  staticFor<H - 1>([&](auto kk) {
+  staticFor<H / 2 - 1>([&](auto kk) {
     constexpr int k = decltype(kk)::value + 1;
     c32 a = z[slot<H>(k)];
     c32 b = z[slot<H>(H - k)];
-    // E = (a + conj b)/2, O = -i (a - conj b)/2, F = E + W_N^k O
+    // E = (a + conj b)/2, O = -i (a - conj b)/2, T = W_N^k O:
+    // F[k] = E + T, F[H-k] = conj(E - T)
     c32 e = c32{0.5f * (a.x + b.x), 0.5f * (a.y - b.y)};
     c32 o = c32{0.5f * (a.y + b.y), -0.5f * (a.x - b.x)};
-    c32 wo = mulRoot<N, k, true>(o);
-    p[k] = cadd(e, wo);
+    c32 t = mulRoot<N, k, true>(o);
+    emit(std::integral_constant<int, k>{}, c32{e.x + t.x, e.y + t.y});
+    emit(std::integral_constant<int, H - k>{}, c32{e.x - t.x, t.y - e.y});
   });
+  if constexpr (H >= 2) {
+    c32 a = z[slot<H>(H / 2)];
+    emit(std::integral_constant<int, H / 2>{}, c32{a.x, -a.y});
+  }
 }
 
-// Inverse of realFixupForward without the 1/2 factors (gain 2): p as above
-// (natural order, p[0] packed) -> z in NATURAL order, ready for an inverse
-// H-point complex FFT whose output z[j] = (x[2j], x[2j+1]) * gain.
 template <int H>
-__device__ __forceinline__ void realFixupInverse(const c32 (&p)[H], c32 (&z)[H]) {
+__device__ __forceinline__ void realFixupForward(const c32 (&z)[H], c32 (&p)[H]) {
+  realFixupForwardEmit<H>(z, [&](auto kk, c32 v) { p[decltype(kk)::value] = v; });
+}
+
+// Inverse of the above without the 1/2 factors (gain 2).  fetch(k) returns F[k]
+// for k = 0..H-1 (k = 0: the packed (F[0], F[H])); z receives, in NATURAL order,
+// the input of an inverse H-point complex FFT whose output is
+// z[j] = (x[2j], x[2j+1]) * gain.
+template <int H, typename Fetch>
+__device__ __forceinline__ void realFixupInverseFetch(Fetch&& fetch, c32 (&z)[H]) {
   constexpr int N = 2 * H;
-  z[0] = c32{p[0].x + p[0].y, p[0].x - p[0].y};
-  staticFor<H - 1>([&](auto kk) {
+  {
+    c32 p0 = fetch(std::integral_constant<int, 0>{});
+    z[0] = c32{p0.x + p0.y, p0.x - p0.y};
+  }
+  staticFor<H / 2 - 1>([&](auto kk) {
     constexpr int k = decltype(kk)::value + 1;
-    c32 a = p[k];
-    c32 b = p[H - k];
-    // E2 = a + conj b, O2 = (a - conj b) W_N^{-k}, Z = E2 + i O2
+    c32 a = fetch(std::integral_constant<int, k>{});
+    c32 b = fetch(std::integral_constant<int, H - k>{});
+    // E2 = a + conj b, O2 = (a - conj b) W_N^{-k}:
+    // Z[k] = E2 + i O2, Z[H-k] = conj(E2) + i conj(O2)
     c32 e = c32{a.x + b.x, a.y - b.y};
     c32 d = c32{a.x - b.x, a.y + b.y};
     c32 o = mulRoot<N, k, false>(d);
     z[k] = c32{e.x - o.y, e.y + o.x};
+    z[H - k] = c32{e.x + o.y, o.x - e.y};
   });
+  if constexpr (H >= 2) {
+    c32 a = fetch(std::integral_constant<int, H / 2>{});
+    z[H / 2] = c32{2.0f * a.x, -2.0f * a.y};
+  }
+}
+
+template <int H>
+__device__ __forceinline__ void realFixupInverse(const c32 (&p)[H], c32 (&z)[H]) {
+  realFixupInverseFetch<H>([&](auto kk) { return p[decltype(kk)::value]; }, z);
 }
 
 }  // namespace fbfft_amd

@@ -19,8 +19,9 @@ def c(a):
 
 
 def rel(a, b):
-    a = np.asarray(a, dtype=np.float64).ravel()
-    b = np.asarray(b, dtype=np.float64).ravel()
+    a, b = np.asarray(a), np.asarray(b)
+    wide = np.complex128 if (np.iscomplexobj(a) or np.iscomplexobj(b)) else np.float64
+    a, b = a.astype(wide).ravel(), b.astype(wide).ravel()
     return float(np.linalg.norm(a - b) / max(np.linalg.norm(b), 1e-300))
 
 
