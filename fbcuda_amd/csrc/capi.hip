@@ -45,6 +45,22 @@ bool okCplx(const fbfft_tensor* t) {
   return aligned(t->data, 8);
 }
 
+// [d0][d1][...][2] -> number of collapsed bins, or -1 if the middle dimensions
+// are not one contiguous run of complex values
+int collapsedBins(const fbfft_tensor* t) {
+  const int d = t->dim;
+  if (d < 3 || d > FBFFT_MAX_DIM) return -1;
+  if (t->size[d - 1] != 2 || t->stride[d - 1] != 1) return -1;
+  long expect = 2, xy = 1;
+  for (int i = d - 2; i >= 2; --i) {
+    if (t->size[i] != 1 && t->stride[i] != expect) return -1;
+    expect *= t->size[i];
+    xy *= t->size[i];
+  }
+  if (d == 3) xy = 1;  // [d0][d1][2]: a single bin
+  return (int)xy;
+}
+
 }  // namespace
 
 extern "C" {
@@ -60,6 +76,30 @@ const char* fbfft_error_string(int code) {
 }
 
 void fbfft_twiddle_table(float* out) { memcpy(out, kTwiddleBits, sizeof(kTwiddleBits)); }
+
+static int run1d(bool forward, const fbfft_tensor* real, const fbfft_tensor* cplx, int padL,
+                 fbfft_stream_t stream) {
+  if (!okTensor(real, 2) || !okTensor(cplx, 3)) return FBFFT_UNSUPPORTED_DIMENSION;
+  const int N = real->size[1];
+  if (!isPow2(N) || N < 2 || N > 256) return FBFFT_UNSUPPORTED_SIZE;
+  if (cplx->size[2] != 2 || cplx->size[1] != N / 2 + 1 || cplx->size[0] != real->size[0])
+    return FBFFT_UNSUPPORTED_DIMENSION;
+  if (padL < 0) return FBFFT_UNSUPPORTED_SIZE;
+  if (!okCplx(cplx)) return FBFFT_UNSUPPORTED_DIMENSION;
+  if (real->size[0] == 0) return FBFFT_SUCCESS;
+  return launchFft1d(forward, N, real->data, real->stride[0], real->stride[1], cplx->data,
+                     cplx->stride[0], cplx->stride[1], real->size[0], padL, stream);
+}
+
+int fbfft_r2c_1d(const fbfft_tensor* real, const fbfft_tensor* cplx, int padL,
+                 fbfft_stream_t stream) {
+  return run1d(true, real, cplx, padL, stream);
+}
+
+int fbfft_c2r_1d(const fbfft_tensor* real, const fbfft_tensor* cplx, int padL,
+                 fbfft_stream_t stream) {
+  return run1d(false, real, cplx, padL, stream);
+}
 
 int fbfft_r2c_2d(const fbfft_tensor* real, const fbfft_tensor* cplx, int padL, int padU,
                  fbfft_stream_t stream) {
@@ -107,14 +147,92 @@ int fbfft_c2r_2d(const fbfft_tensor* cplx, const fbfft_tensor* real, int padL, i
 
 }  // extern "C"
 
+extern "C" int fbfft_transpose_mm(const fbfft_tensor* A, const fbfft_tensor* B,
+                                  const fbfft_tensor* C, int conjA, int conjB, int accumulate,
+                                  float invNorm, fbfft_stream_t stream) {
+  if (!A || !B || !C) return FBFFT_UNSUPPORTED_DIMENSION;
+  if (conjA && conjB) return FBFFT_UNSUPPORTED_DIMENSION;  // no reference role uses both
+  const int xa = collapsedBins(A), xb = collapsedBins(B), xc = collapsedBins(C);
+  if (xa < 0 || xb < 0 || xc < 0 || xa != xb || xa != xc) return FBFFT_UNSUPPORTED_DIMENSION;
+  const int I = conjA ? A->size[1] : A->size[0];
+  const int K = conjA ? A->size[0] : A->size[1];
+  const int Kb = conjB ? B->size[1] : B->size[0];
+  const int J = conjB ? B->size[0] : B->size[1];
+  if (K != Kb || C->size[0] != I || C->size[1] != J) return FBFFT_UNSUPPORTED_DIMENSION;
+  const fbfft_tensor* ts[3] = {A, B, C};
+  for (const fbfft_tensor* t : ts) {
+    if (t->stride[0] % 2 != 0 || t->stride[1] % 2 != 0 || !aligned(t->data, 8))
+      return FBFFT_UNSUPPORTED_DIMENSION;
+  }
+  return launchTransposeMM(A->data, A->stride[0], A->stride[1], B->data, B->stride[0],
+                           B->stride[1], C->data, C->stride[0], C->stride[1], I, J, K, xa,
+                           conjA != 0, conjB != 0, accumulate != 0, invNorm, stream);
+}
+
+namespace {
+size_t specFloats(int planes, int N) { return (size_t)planes * (N / 2 + 1) * N * 2; }
+
+// [d0][d1][h][w] -> [d0*d1][h][w] when the two leading dimensions collapse
+bool collapse4(const fbfft_tensor* t, RealView* v) {
+  if (t->size[0] > 1 && t->stride[0] != (long)t->stride[1] * t->size[1]) return false;
+  *v = RealView{t->data, t->stride[1], t->stride[2], t->stride[3],
+                t->size[0] * t->size[1], t->size[2], t->size[3]};
+  return true;
+}
+}  // namespace
+
+extern "C" size_t fbfft_conv_fprop_workspace(int batch, int cin, int cout, int fftSize) {
+  if (batch <= 0 || cin <= 0 || cout <= 0) return 0;
+  const size_t fl = specFloats(batch * cin, fftSize) + specFloats(cout * cin, fftSize) +
+                    specFloats(batch * cout, fftSize);
+  return fl * sizeof(float);
+}
+
+extern "C" int fbfft_conv_fprop(const fbfft_tensor* input, const fbfft_tensor* weight,
+                                const fbfft_tensor* output, int fftSize, void* workspace,
+                                size_t workspaceBytes, fbfft_stream_t stream) {
+  if (!okTensor(input, 4) || !okTensor(weight, 4) || !okTensor(output, 4))
+    return FBFFT_UNSUPPORTED_DIMENSION;
+  const int N = fftSize;
+  if (!(N == 8 || N == 16 || N == 32)) return FBFFT_UNSUPPORTED_SIZE;
+  const int B = input->size[0], Cin = input->size[1], H = input->size[2], W = input->size[3];
+  const int Cout = weight->size[0], kH = weight->size[2], kW = weight->size[3];
+  if (weight->size[1] != Cin || output->size[0] != B || output->size[1] != Cout)
+    return FBFFT_UNSUPPORTED_DIMENSION;
+  if (H > N || W > N || kH > H || kW > W) return FBFFT_UNSUPPORTED_SIZE;
+  if (output->size[2] != H - kH + 1 || output->size[3] != W - kW + 1)
+    return FBFFT_UNSUPPORTED_DIMENSION;
+  if (empty(input) || empty(weight) || empty(output)) return FBFFT_SUCCESS;
+  if (!workspace || !aligned(workspace, 256) ||
+      workspaceBytes < fbfft_conv_fprop_workspace(B, Cin, Cout, N))
+    return FBFFT_UNSUPPORTED_DIMENSION;
+  RealView in, wt, out;
+  if (!collapse4(input, &in) || !collapse4(weight, &wt) || !collapse4(output, &out))
+    return FBFFT_UNSUPPORTED_DIMENSION;
+
+  const int rows = N / 2 + 1;
+  const int plane = rows * N * 2;  // floats per spectrum plane
+  float* inSpec = static_cast<float*>(workspace);
+  float* wtSpec = inSpec + specFloats(B * Cin, N);
+  float* outSpec = wtSpec + specFloats(Cout * Cin, N);
+  auto spec = [&](float* p, int planes) { return CplxView{p, plane, 2 * N, 2, planes, rows, N}; };
+
+  int rc = launchFft2dSmallForward(N, in, spec(inSpec, B * Cin), 0, 0, stream);
+  if (rc != FBFFT_SUCCESS) return rc;
+  rc = launchFft2dSmallForward(N, wt, spec(wtSpec, Cout * Cin), 0, 0, stream);
+  if (rc != FBFFT_SUCCESS) return rc;
+  // o(b, f) = sum_p i(b, p) . conj(w(f, p)), scaled by 1/N^2 (MM-inl.cuh:193-196)
+  rc = launchTransposeMM(inSpec, (long)Cin * plane, plane, wtSpec, (long)Cin * plane, plane,
+                         outSpec, (long)Cout * plane, plane, B, Cout, Cin, rows * N, false, true,
+                         false, 1.0f / (float)(N * N), stream);
+  if (rc != FBFFT_SUCCESS) return rc;
+  // the valid region is the top-left corner of the inverse transform: crop on store
+  return launchFft2dSmallInverse(N, spec(outSpec, B * Cout), out, 0, 0, stream);
+}
+
 // ---- entry points whose kernels are not wired yet ----
 extern "C" {
-int fbfft_r2c_1d(const fbfft_tensor*, const fbfft_tensor*, int, fbfft_stream_t) { return FBFFT_UNSUPPORTED_SIZE; }
-int fbfft_c2r_1d(const fbfft_tensor*, const fbfft_tensor*, int, fbfft_stream_t) { return FBFFT_UNSUPPORTED_SIZE; }
 int fbfft_c2c_2d_pass2(const fbfft_tensor*, const fbfft_tensor*, fbfft_stream_t) { return FBFFT_UNSUPPORTED_SIZE; }
 int fbfft_c2c_2d_inverse_pass1(const fbfft_tensor*, const fbfft_tensor*, fbfft_stream_t) { return FBFFT_UNSUPPORTED_SIZE; }
-int fbfft_transpose_mm(const fbfft_tensor*, const fbfft_tensor*, const fbfft_tensor*, int, int, int, float, fbfft_stream_t) { return FBFFT_UNSUPPORTED_SIZE; }
 int fbfft_iterated_conv(int, const fbfft_tile*, const fbfft_tile*, const fbfft_tensor*, int, float, int, size_t, fbfft_stream_t) { return 0; }
-size_t fbfft_conv_fprop_workspace(int, int, int, int) { return 0; }
-int fbfft_conv_fprop(const fbfft_tensor*, const fbfft_tensor*, const fbfft_tensor*, int, void*, size_t, fbfft_stream_t) { return FBFFT_UNSUPPORTED_SIZE; }
 }

@@ -46,4 +46,11 @@ int launchFft2dLargeForward(int N, const RealView& real, const CplxView& cplx, i
 int launchFft2dLargeInverse(int N, const CplxView& cplx, const RealView& real, int padL, int padU,
                             hipStream_t s);
 
+int launchFft1d(bool forward, int N, float* real, int sb, int sx, float* cplx, int cb, int ck,
+                int B, int padL, hipStream_t s);
+
+int launchTransposeMM(const float* A, long a0, long a1, const float* B, long b0, long b1, float* C,
+                      long c0, long c1, int I, int J, int K, int XY, bool conjA, bool conjB,
+                      bool accumulate, float invNorm, hipStream_t s);
+
 }  // namespace fbfft_amd

@@ -22,6 +22,7 @@
 //      16-byte stores; the packed column is unpacked on the way out.
 // The inverse runs the same steps backwards and crops on store.
 #include "common.h"
+#include "fft_lds.h"
 #include "fft_regs.h"
 
 namespace fbfft_amd {
@@ -43,56 +44,6 @@ struct LargeCfg {
   static constexpr int F4_CPLX = (H + 1) * N / 2;     // float4 per spectrum plane
 };
 
-// full-circle twiddles e^{-/+ 2 pi i m / 256}, m = 0..255, from the half-circle table
-template <bool FWD, int THREADS>
-__device__ __forceinline__ void fillTwiddles(c32* tw, int t) {
-  for (int m = t; m < 256; m += THREADS) {
-    const int h = m & 127;
-    float c = __builtin_bit_cast(float, kTwiddleBits[2 * h]);
-    float s = __builtin_bit_cast(float, kTwiddleBits[2 * h + 1]);
-    if (m >= 128) {
-      c = -c;
-      s = -s;
-    }
-    tw[m] = c32{c, FWD ? -s : s};
-  }
-}
-
-// Lane g of G computes outputs X[G*k + g], k = 0..N/G-1, of the N-point FFT of
-// col[0..N) (LDS, unit stride); they are left in v[slot<N/G>(k)].
-template <int N, int G, bool FWD>
-__device__ __forceinline__ void splitColumnFFT(const c32* col, int g, const c32* tw,
-                                               c32 (&v)[N / G]) {
-  constexpr int L = N / G;
-  static_assert(G == 2 || G == 4, "column split");
-  if constexpr (G == 2) {
-    const float sgn = g ? -1.0f : 1.0f;
-    staticFor<L>([&](auto jj) {
-      constexpr int j = decltype(jj)::value;
-      c32 u0 = col[j], u1 = col[j + L];
-      c32 comb = c32{u0.x + sgn * u1.x, u0.y + sgn * u1.y};
-      c32 w = tw[(g * (j * (256 / N))) & 255];
-      v[j] = cmul(comb, w);
-    });
-  } else {
-    const float sA = (g & 1) ? -1.0f : 1.0f;
-    const bool rot = (g & 1) != 0;
-    // forward: omega = -i  -> g=1: -i*b, g=3: +i*b;  inverse: the other way round
-    const float sB = (g == 0) ? 1.0f : (g == 2) ? -1.0f : ((g == 1) == FWD) ? -1.0f : 1.0f;
-    staticFor<L>([&](auto jj) {
-      constexpr int j = decltype(jj)::value;
-      c32 u0 = col[j], u1 = col[j + L], u2 = col[j + 2 * L], u3 = col[j + 3 * L];
-      c32 a = c32{u0.x + sA * u2.x, u0.y + sA * u2.y};
-      c32 b = c32{u1.x + sA * u3.x, u1.y + sA * u3.y};
-      c32 br = rot ? c32{-b.y, b.x} : b;  // i*b when rot
-      c32 comb = c32{a.x + sB * br.x, a.y + sB * br.y};
-      c32 w = tw[(g * (j * (256 / N))) & 255];
-      v[j] = cmul(comb, w);
-    });
-  }
-  difFFT<L, FWD>(v);
-}
-
 template <int N, bool FAST_REAL, bool FAST_CPLX>
 __global__ __launch_bounds__(LargeCfg<N>::THREADS) void fft2dLargeForward(RealView real,
                                                                          CplxView cplx, int padL,
@@ -103,7 +54,7 @@ __global__ __launch_bounds__(LargeCfg<N>::THREADS) void fft2dLargeForward(RealVi
   __shared__ __align__(8) c32 tw[256];
   const int t = threadIdx.x;
   const int b = blockIdx.x;
-  fillTwiddles<true, THREADS>(tw, t);
+  fillTwiddles<true>(tw, t, THREADS);
 
   // ---- 1. real plane -> LDS [y][x] ----
   if constexpr (FAST_REAL) {
@@ -152,7 +103,7 @@ __global__ __launch_bounds__(LargeCfg<N>::THREADS) void fft2dLargeForward(RealVi
   // ---- 4. column pass ----
   const int col = t % H, g = t / H;
   c32 v[L];
-  splitColumnFFT<N, G, true>(cb + col * CS, g, tw, v);
+  splitFFT<N, G, true>(cb + col * CS, g, tw, v);
   __syncthreads();  // all columns consumed
   // ---- 5. [kx][ky] back to LDS ----
   staticFor<L>([&](auto kk) {
@@ -205,7 +156,7 @@ __global__ __launch_bounds__(LargeCfg<N>::THREADS) void fft2dLargeInverse(CplxVi
   __shared__ __align__(8) c32 tw[256];
   const int t = threadIdx.x;
   const int b = blockIdx.x;
-  fillTwiddles<false, THREADS>(tw, t);
+  fillTwiddles<false>(tw, t, THREADS);
   c32* cb = reinterpret_cast<c32*>(buf);
 
   // ---- copy in [kx][ky]; row H is folded into row 0: Z = F0 + i*FH ----
@@ -251,7 +202,7 @@ __global__ __launch_bounds__(LargeCfg<N>::THREADS) void fft2dLargeInverse(CplxVi
   // ---- column pass (inverse) ----
   const int col = t % H, g = t / H;
   c32 v[L];
-  splitColumnFFT<N, G, false>(cb + col * CS, g, tw, v);
+  splitFFT<N, G, false>(cb + col * CS, g, tw, v);
   __syncthreads();
   // [y][kx]
   staticFor<L>([&](auto kk) {

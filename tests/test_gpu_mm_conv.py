@@ -1,0 +1,132 @@
+"""GPU parity of transposeMM (C ABI fbfft_transpose_mm) and of the FFT convolution
+forward pass built from the primitives (fbfft_conv_fprop)."""
+import numpy as np
+import pytest
+import torch
+
+import fbcuda_amd as F
+from fbcuda_amd import synth
+from gpu_util import TOL_CONV, TOL_FFT, dev, rel
+
+pytestmark = pytest.mark.gpu
+
+
+def mm(A, B, conjA, conjB, invNorm, C0=None):
+    Ad = torch.from_numpy(A).to(dev())
+    Bd = torch.from_numpy(B).to(dev())
+    I = A.shape[1] if conjA else A.shape[0]
+    J = B.shape[0] if conjB else B.shape[1]
+    if C0 is None:
+        Cd = torch.full((I, J) + A.shape[2:], float("nan"), device=dev())
+    else:
+        Cd = torch.from_numpy(C0).to(dev())
+    rc = F.transposeMM(Ad, Bd, Cd, invNorm, conjA, conjB, C0 is not None)
+    torch.cuda.synchronize()
+    return rc, Cd.cpu().numpy()
+
+
+ROLES = [(False, True), (True, False), (False, False)]  # updateOutput, accGrad, updateGradInput
+
+
+@pytest.mark.parametrize("conjA,conjB", ROLES)
+@pytest.mark.parametrize("I,J,K,shape", [
+    (32, 32, 4, (5, 8)),        # one tile, xy = 40 (N = 8 spectra)
+    (64, 96, 16, (9, 16)),      # N = 16 spectra
+    (33, 7, 5, (17, 32)),       # ragged I/J/K, xy = 544
+    (1, 3, 3, (5, 8)),          # batch 1, RGB-like reduction
+    (40, 70, 64, (3, 2)),       # xy = 6: partial bin chunk
+])
+def test_mm_vs_oracle(oracle, conjA, conjB, I, J, K, shape):
+    xy = shape[0] * shape[1]
+    A = synth.normal(((K, I) if conjA else (I, K)) + shape + (2,), seed=1).numpy()
+    B = synth.normal(((J, K) if conjB else (K, J)) + shape + (2,), seed=2).numpy()
+    rc, got = mm(A, B, conjA, conjB, 0.125)
+    assert rc == F.Success
+    A3 = A.reshape(A.shape[0], A.shape[1], xy, 2)
+    B3 = B.reshape(B.shape[0], B.shape[1], xy, 2)
+    want32 = oracle.transpose_mm(A3, B3, conjA, conjB, 0.125)
+    want64 = oracle.transpose_mm64(A3, B3, conjA, conjB, 0.125)
+    got3 = got.reshape(I, J, xy, 2)
+    assert rel(got3, want32) < TOL_FFT
+    assert rel(got3, want64) < TOL_FFT
+    # Accumulate: invNorm scales the accumulated-into value as well (MM-inl.cuh:322-324)
+    C0 = synth.normal((I, J) + shape + (2,), seed=3).numpy()
+    rc, acc = mm(A, B, conjA, conjB, 0.125, C0=C0)
+    assert rc == F.Success
+    want_acc = oracle.transpose_mm(A3, B3, conjA, conjB, 0.125, C=C0.reshape(I, J, xy, 2))
+    assert rel(acc.reshape(I, J, xy, 2), want_acc) < TOL_FFT
+
+
+def test_mm_rank3_rank4_and_errors():
+    d = dev()
+    A = torch.zeros((4, 6, 40, 2), device=d)
+    B = torch.zeros((5, 6, 40, 2), device=d)
+    C = torch.zeros((4, 5, 40, 2), device=d)
+    assert F.transposeMM(A, B, C, 1.0, False, True) == F.Success
+    assert F.transposeMM(A, B, torch.zeros((4, 6, 40, 2), device=d), 1.0, False, True) == F.UnsupportedDimension
+    assert F.transposeMM(A, B, C, 1.0, False, False) == F.UnsupportedDimension  # K mismatch
+    assert F.transposeMM(A, B[:, :, ::2], C, 1.0, False, True) == F.UnsupportedDimension  # strided xy
+    assert F.transposeMM(A[..., 0], B[..., 0], C[..., 0], 1.0, False, True) == F.UnsupportedDimension
+    torch.cuda.synchronize()
+
+
+def test_mm_config3_shape_subset(oracle):
+    """configs[3] contraction shape (128 x 64 x 192 over 544 bins): full GPU run,
+    fp64 check on a seeded subset of (i, j) pairs."""
+    d = dev()
+    I, K, J, xy = 128, 64, 192, 544
+    A = synth.normal((I, K, 17, 32, 2), seed=30, device=d)
+    B = synth.normal((J, K, 17, 32, 2), seed=31, device=d)
+    C = torch.empty((I, J, 17, 32, 2), device=d)
+    assert F.transposeMM(A, B, C, 1.0 / 1024, False, True) == F.Success
+    torch.cuda.synchronize()
+    ii = [0, 5, 31, 32, 77, 127]
+    jj = [0, 1, 63, 64, 100, 191]
+    want = oracle.transpose_mm64(A[ii].cpu().numpy().reshape(len(ii), K, xy, 2),
+                                 B[jj].cpu().numpy().reshape(len(jj), K, xy, 2), False, True, 1.0 / 1024)
+    got = C[ii][:, jj].cpu().numpy().reshape(len(ii), len(jj), xy, 2)
+    assert rel(got, want) < TOL_FFT
+
+
+def conv(x, w, N):
+    d = dev()
+    xd, wd = torch.from_numpy(x).to(d), torch.from_numpy(w).to(d)
+    Bn, Cin, H, W = x.shape
+    Cout, _, kH, kW = w.shape
+    out = torch.full((Bn, Cout, H - kH + 1, W - kW + 1), float("nan"), device=d)
+    ws = torch.empty(F.conv_fprop_workspace(Bn, Cin, Cout, N), dtype=torch.uint8, device=d)
+    rc = F.conv_fprop(xd, wd, out, N, ws)
+    torch.cuda.synchronize()
+    return rc, out.cpu().numpy()
+
+
+@pytest.mark.parametrize("N,H,W,k,Bn,Cin,Cout", [
+    (8, 8, 8, 3, 2, 3, 4), (16, 13, 16, 5, 3, 5, 7), (32, 27, 27, 5, 4, 8, 6), (32, 32, 30, 1, 2, 2, 2)])
+def test_conv_fprop_small(oracle, N, H, W, k, Bn, Cin, Cout):
+    x = synth.normal((Bn, Cin, H, W), seed=30).numpy()
+    w = synth.normal((Cout, Cin, k, k), seed=31, std=0.02).numpy()
+    rc, got = conv(x, w, N)
+    assert rc == F.Success
+    assert rel(got, oracle.corr2d_valid(x, w)) < TOL_CONV
+
+
+def test_conv_fprop_config3(oracle):
+    """configs[3]: 128x64x27x27 * 192x64x5x5 -> 128x192x23x23; fp64 direct
+    correlation on 4096 seeded output pixels plus two whole (n, f) planes."""
+    d = dev()
+    x = synth.normal((128, 64, 27, 27), seed=30, device=d)
+    w = synth.normal((192, 64, 5, 5), seed=31, std=0.02, device=d)
+    out = torch.full((128, 192, 23, 23), float("nan"), device=d)
+    ws = torch.empty(F.conv_fprop_workspace(128, 64, 192, 32), dtype=torch.uint8, device=d)
+    assert F.conv_fprop(x, w, out, 32, ws) == F.Success
+    torch.cuda.synchronize()
+    assert bool(torch.isfinite(out).all())
+    rng = np.random.default_rng(33)
+    coords = np.stack([rng.integers(0, 128, 4096), rng.integers(0, 192, 4096),
+                       rng.integers(0, 23, 4096), rng.integers(0, 23, 4096)], axis=1).astype(np.int32)
+    xh, wh, oh = x.cpu().numpy(), w.cpu().numpy(), out.cpu().numpy()
+    want = oracle.corr2d_valid_at(xh, wh, coords)
+    got = oh[coords[:, 0], coords[:, 1], coords[:, 2], coords[:, 3]]
+    assert rel(got, want) < TOL_CONV
+    full = oracle.corr2d_valid(xh[[0, 127]], wh[[0, 191]])
+    assert rel(oh[[0, 127]][:, [0, 191]], full) < TOL_CONV
