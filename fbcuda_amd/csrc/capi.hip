@@ -234,5 +234,11 @@ extern "C" int fbfft_conv_fprop(const fbfft_tensor* input, const fbfft_tensor* w
 extern "C" {
 int fbfft_c2c_2d_pass2(const fbfft_tensor*, const fbfft_tensor*, fbfft_stream_t) { return FBFFT_UNSUPPORTED_SIZE; }
 int fbfft_c2c_2d_inverse_pass1(const fbfft_tensor*, const fbfft_tensor*, fbfft_stream_t) { return FBFFT_UNSUPPORTED_SIZE; }
-int fbfft_iterated_conv(int, const fbfft_tile*, const fbfft_tile*, const fbfft_tensor*, int, float, int, size_t, fbfft_stream_t) { return 0; }
+int fbfft_iterated_conv(int fftSize, const fbfft_tile* ins, const fbfft_tile* outs,
+                        const fbfft_tensor* weight, int pass, float scale, int batchSize,
+                        size_t numTiles, fbfft_stream_t stream) {
+  if (!okTensor(weight, 4) || !ins || !outs) return 0;
+  return launchIteratedConv(fftSize, ins, outs, weight->data, weight->stride, weight->size, pass,
+                            scale, batchSize, numTiles, stream);
+}
 }

@@ -53,4 +53,8 @@ int launchTransposeMM(const float* A, long a0, long a1, const float* B, long b0,
                       long c0, long c1, int I, int J, int K, int XY, bool conjA, bool conjB,
                       bool accumulate, float invNorm, hipStream_t s);
 
+int launchIteratedConv(int N, const fbfft_tile* ins, const fbfft_tile* outs, float* weight,
+                       const int* wStride, const int* wSize, int pass, float scale, int batch,
+                       size_t numTiles, hipStream_t s);
+
 }  // namespace fbfft_amd

@@ -1,0 +1,127 @@
+// Per-plane passes of the N <= 32 2D transforms, shared by the stand-alone
+// kernels and by the fused tiled convolution.  A plane is handled by T = N/2
+// lanes of one wave; lane l owns columns 2l, 2l+1 in the column pass and packed
+// spectral row l in the row pass.  The plane buffer in LDS holds N/2 (+1) rows of
+// N complex with row stride N + 2 (rows stay 16-byte aligned and consecutive rows
+// start 4 banks apart, so 16-byte accesses by the lanes of a plane do not
+// conflict).  Packed row 0 carries spectral rows 0 and N/2 (both real along the
+// column axis) as real and imaginary part.  Callers place the barriers.
+#pragma once
+
+#include "common.h"
+#include "fft_regs.h"
+
+namespace fbfft_amd {
+
+template <int N>
+struct PlaneCfg {
+  static constexpr int H = N / 2;
+  static constexpr int T = N / 2;     // lanes per plane
+  static constexpr int RS = N + 2;    // LDS row stride (complex)
+};
+
+__device__ __forceinline__ float4 ldsLoad4(const c32* p) {
+  return *reinterpret_cast<const float4*>(p);
+}
+__device__ __forceinline__ void ldsStore4(c32* p, c32 a, c32 b) {
+  *reinterpret_cast<float4*>(p) = float4{a.x, a.y, b.x, b.y};
+}
+
+// Two columns of a real plane through a bounds-checked strided view:
+// z[j] = (X[2j][x], X[2j+1][x]) for x = 2l and 2l+1, zero outside the window
+// (the padding rule of MemoryAccess.cuh:19-25).
+template <int N>
+__device__ __forceinline__ void loadColumnsWindow(const float* src, int sy, int sx, int h, int w,
+                                                  int padL, int padU, int l, c32 (&z0)[N / 2],
+                                                  c32 (&z1)[N / 2]) {
+  const int x0 = 2 * l, x1 = 2 * l + 1;
+  auto fetch = [&](int y, int x) {
+    return inWindow(y, x, padU, padL, h, w)
+               ? src[(size_t)(y - padU) * sy + (size_t)(x - padL) * sx] : 0.0f;
+  };
+  staticFor<N / 2>([&](auto jj) {
+    constexpr int j = decltype(jj)::value;
+    z0[j] = c32{fetch(2 * j, x0), fetch(2 * j + 1, x0)};
+    z1[j] = c32{fetch(2 * j, x1), fetch(2 * j + 1, x1)};
+  });
+}
+
+// Column pass (forward): N/2-point FFTs of the two packed columns, real-input
+// fix-up, packed rows written to the plane buffer.
+template <int N>
+__device__ __forceinline__ void columnPassForward(c32 (&z0)[N / 2], c32 (&z1)[N / 2], c32* plane,
+                                                  int l) {
+  constexpr int H = N / 2, RS = PlaneCfg<N>::RS;
+  difFFT<H, true>(z0);
+  difFFT<H, true>(z1);
+  c32 p0[H], p1[H];
+  realFixupForward<H>(z0, p0);
+  realFixupForward<H>(z1, p1);
+  c32* dst = plane + 2 * l;
+  staticFor<H>([&](auto rr) {
+    constexpr int r = decltype(rr)::value;
+    ldsStore4(dst + r * RS, p0[r], p1[r]);
+  });
+}
+
+// Row pass: lane l transforms packed row l in place (natural order in and out).
+template <int N, bool FWD>
+__device__ __forceinline__ void rowPassInPlace(c32* plane, int l) {
+  constexpr int RS = PlaneCfg<N>::RS;
+  c32 row[N];
+  c32* p = plane + l * RS;
+  staticFor<N / 2>([&](auto jj) {
+    constexpr int j = decltype(jj)::value;
+    float4 v = ldsLoad4(p + 2 * j);
+    row[2 * j] = c32{v.x, v.y};
+    row[2 * j + 1] = c32{v.z, v.w};
+  });
+  difFFT<N, FWD>(row);
+  staticFor<N / 2>([&](auto jj) {
+    constexpr int j = decltype(jj)::value;
+    ldsStore4(p + 2 * j, row[slot<N>(2 * j)], row[slot<N>(2 * j + 1)]);
+  });
+}
+
+// Column pass (inverse): reads packed rows of columns 2l, 2l+1, undoes the
+// real-input fix-up and runs the inverse N/2-point FFTs.  On return
+// z[slot<N/2>(j)] = (X[2j][x], X[2j+1][x]) * N*N for the two columns.
+template <int N>
+__device__ __forceinline__ void columnPassInverse(const c32* plane, int l, c32 (&z0)[N / 2],
+                                                  c32 (&z1)[N / 2]) {
+  constexpr int H = N / 2, RS = PlaneCfg<N>::RS;
+  c32 p0[H], p1[H];
+  const c32* src = plane + 2 * l;
+  staticFor<H>([&](auto rr) {
+    constexpr int r = decltype(rr)::value;
+    float4 v = ldsLoad4(src + r * RS);
+    p0[r] = c32{v.x, v.y};
+    p1[r] = c32{v.z, v.w};
+  });
+  realFixupInverse<H>(p0, z0);
+  realFixupInverse<H>(p1, z1);
+  difFFT<H, false>(z0);
+  difFFT<H, false>(z1);
+}
+
+// Two columns of results through a bounds-checked strided view (crop on store).
+template <int N>
+__device__ __forceinline__ void storeColumnsWindow(float* dst, int sy, int sx, int h, int w, int padL,
+                                                   int padU, int l, const c32 (&z0)[N / 2],
+                                                   const c32 (&z1)[N / 2], float scale) {
+  const int x0 = 2 * l, x1 = 2 * l + 1;
+  auto put = [&](int y, int x, float v) {
+    if (inWindow(y, x, padU, padL, h, w))
+      dst[(size_t)(y - padU) * sy + (size_t)(x - padL) * sx] = v * scale;
+  };
+  staticFor<N / 2>([&](auto jj) {
+    constexpr int j = decltype(jj)::value;
+    c32 a = z0[slot<N / 2>(j)], c = z1[slot<N / 2>(j)];
+    put(2 * j, x0, a.x);
+    put(2 * j, x1, c.x);
+    put(2 * j + 1, x0, a.y);
+    put(2 * j + 1, x1, c.y);
+  });
+}
+
+}  // namespace fbfft_amd

@@ -18,6 +18,7 @@
 // The inverse runs the same steps backwards.  Each plane crosses HBM exactly
 // once in each direction: 4N^2 + 8N(N/2+1) bytes.
 #include "common.h"
+#include "fft2d_core.h"
 #include "fft_regs.h"
 
 namespace fbfft_amd {
@@ -29,21 +30,13 @@ struct SmallCfg {
   static constexpr int T = N / 2;          // lanes per plane
   static constexpr int P = 64 / T;         // planes per wave
   static constexpr int ROWS = H + 1;       // spectral rows kept in LDS
-  static constexpr int RS = N + 2;         // LDS row stride (complex): 16-byte aligned rows,
-                                           // consecutive rows start 4 (mod 64) banks apart
+  static constexpr int RS = PlaneCfg<N>::RS;  // LDS row stride (complex)
   static constexpr int PS = ROWS * RS + (N == 8 ? 2 : 0);  // LDS plane stride (complex)
   static constexpr int F4_PER_PLANE = ROWS * N / 2;        // float4 per spectrum plane
   static constexpr int ITERS = P * F4_PER_PLANE / 64;      // float4 per lane per wave
   static_assert(P * F4_PER_PLANE % 64 == 0, "copy loop must divide evenly");
   static_assert(RS % 2 == 0 && PS % 2 == 0, "rows must stay 16-byte aligned");
 };
-
-__device__ __forceinline__ float4 ldsLoad4(const c32* p) {
-  return *reinterpret_cast<const float4*>(p);
-}
-__device__ __forceinline__ void ldsStore4(c32* p, c32 a, c32 b) {
-  *reinterpret_cast<float4*>(p) = float4{a.x, a.y, b.x, b.y};
-}
 
 // FAST_REAL: real is [B][N][N] with unit x stride, even row/batch strides,
 //            8-byte aligned base and zero padding -> 8-byte vector accesses.
@@ -75,51 +68,15 @@ __global__ __launch_bounds__(64) void fft2dSmallForward(RealView real, CplxView 
       z1[j] = c32{r0.y, r1.y};
     });
   } else {
-    const float* src = real.data + (size_t)b * real.sb;
-    const int x0 = 2 * l, x1 = 2 * l + 1;
-    auto fetch = [&](int y, int x) {
-      return inWindow(y, x, padU, padL, real.h, real.w)
-                 ? src[(size_t)(y - padU) * real.sy + (size_t)(x - padL) * real.sx] : 0.0f;
-    };
-    staticFor<H>([&](auto jj) {
-      constexpr int j = decltype(jj)::value;
-      z0[j] = c32{fetch(2 * j, x0), fetch(2 * j + 1, x0)};
-      z1[j] = c32{fetch(2 * j, x1), fetch(2 * j + 1, x1)};
-    });
+    loadColumnsWindow<N>(real.data + (size_t)b * real.sb, real.sy, real.sx, real.h, real.w, padL,
+                         padU, l, z0, z1);
   }
-  difFFT<H, true>(z0);
-  difFFT<H, true>(z1);
-  {
-    c32 p0[H], p1[H];
-    realFixupForward<H>(z0, p0);
-    realFixupForward<H>(z1, p1);
-    c32* dst = lds + pl * PS + 2 * l;
-    staticFor<H>([&](auto rr) {
-      constexpr int r = decltype(rr)::value;
-      ldsStore4(dst + r * RS, p0[r], p1[r]);
-    });
-  }
+  c32* plane = lds + pl * PS;
+  columnPassForward<N>(z0, z1, plane, l);
   __syncthreads();
 
   // ---- row pass: lane l owns packed row l ----
-  c32 row[N];
-  {
-    const c32* src = lds + pl * PS + l * RS;
-    staticFor<N / 2>([&](auto jj) {
-      constexpr int j = decltype(jj)::value;
-      float4 v = ldsLoad4(src + 2 * j);
-      row[2 * j] = c32{v.x, v.y};
-      row[2 * j + 1] = c32{v.z, v.w};
-    });
-  }
-  difFFT<N, true>(row);
-  {
-    c32* dst = lds + pl * PS + l * RS;
-    staticFor<N / 2>([&](auto jj) {
-      constexpr int j = decltype(jj)::value;
-      ldsStore4(dst + 2 * j, row[slot<N>(2 * j)], row[slot<N>(2 * j + 1)]);
-    });
-  }
+  rowPassInPlace<N, true>(plane, l);
   __syncthreads();
 
   // ---- copy out: (H+1) x N complex per plane, rows 0 and H unpacked from packed row 0 ----
@@ -210,42 +167,13 @@ __global__ __launch_bounds__(64) void fft2dSmallInverse(CplxView cplx, RealView 
   __syncthreads();
 
   // ---- row pass (inverse) ----
-  c32 row[N];
-  {
-    const c32* src = lds + pl * PS + l * RS;
-    staticFor<N / 2>([&](auto jj) {
-      constexpr int j = decltype(jj)::value;
-      float4 v = ldsLoad4(src + 2 * j);
-      row[2 * j] = c32{v.x, v.y};
-      row[2 * j + 1] = c32{v.z, v.w};
-    });
-  }
-  difFFT<N, false>(row);
-  {
-    c32* dst = lds + pl * PS + l * RS;
-    staticFor<N / 2>([&](auto jj) {
-      constexpr int j = decltype(jj)::value;
-      ldsStore4(dst + 2 * j, row[slot<N>(2 * j)], row[slot<N>(2 * j + 1)]);
-    });
-  }
+  c32* plane = lds + pl * PS;
+  rowPassInPlace<N, false>(plane, l);
   __syncthreads();
 
   // ---- column pass (inverse): lane l owns columns 2l, 2l+1 ----
-  c32 p0[H], p1[H];
-  {
-    const c32* src = lds + pl * PS + 2 * l;
-    staticFor<H>([&](auto rr) {
-      constexpr int r = decltype(rr)::value;
-      float4 v = ldsLoad4(src + r * RS);
-      p0[r] = c32{v.x, v.y};
-      p1[r] = c32{v.z, v.w};
-    });
-  }
   c32 z0[H], z1[H];
-  realFixupInverse<H>(p0, z0);
-  realFixupInverse<H>(p1, z1);
-  difFFT<H, false>(z0);
-  difFFT<H, false>(z1);
+  columnPassInverse<N>(plane, l, z0, z1);
 
   const int b = b0 + pl;
   if (b >= B) return;
@@ -259,20 +187,8 @@ __global__ __launch_bounds__(64) void fft2dSmallInverse(CplxView cplx, RealView 
       dst[(size_t)(2 * j + 1) * rs2] = float2{a.y, c.y};
     });
   } else {
-    float* dst = real.data + (size_t)b * real.sb;
-    const int x0 = 2 * l, x1 = 2 * l + 1;
-    auto put = [&](int y, int x, float v) {
-      if (inWindow(y, x, padU, padL, real.h, real.w))
-        dst[(size_t)(y - padU) * real.sy + (size_t)(x - padL) * real.sx] = v;
-    };
-    staticFor<H>([&](auto jj) {
-      constexpr int j = decltype(jj)::value;
-      c32 a = z0[slot<H>(j)], c = z1[slot<H>(j)];
-      put(2 * j, x0, a.x);
-      put(2 * j, x1, c.x);
-      put(2 * j + 1, x0, a.y);
-      put(2 * j + 1, x1, c.y);
-    });
+    storeColumnsWindow<N>(real.data + (size_t)b * real.sb, real.sy, real.sx, real.h, real.w, padL,
+                          padU, l, z0, z1, 1.0f);
   }
 }
 
