@@ -124,7 +124,9 @@ int fbfft_r2c_2d(const fbfft_tensor* real, const fbfft_tensor* cplx, int padL, i
   if (N <= 32) return launchFft2dSmallForward(N, realView3(real), cplxView4(cplx), padL, padU, stream);
   if (!scratchForm)
     return launchFft2dLargeForward(N, realView3(real), cplxView4(cplx), padL, padU, stream);
-  return FBFFT_UNSUPPORTED_SIZE;
+  return launchTwoPass(N, 0, real->data, real->stride[0], real->stride[1], real->stride[2],
+                       cplx->data, cplx->stride[0], cplx->stride[1], cplx->stride[2],
+                       real->size[0], real->size[1], real->size[2], padL, padU, stream);
 }
 
 int fbfft_c2r_2d(const fbfft_tensor* cplx, const fbfft_tensor* real, int padL, int padU,
@@ -142,7 +144,9 @@ int fbfft_c2r_2d(const fbfft_tensor* cplx, const fbfft_tensor* real, int padL, i
   if (empty(real) || empty(cplx)) return FBFFT_SUCCESS;
   if (N <= 32) return launchFft2dSmallInverse(N, cplxView4(cplx), realView3(real), padL, padU, stream);
   if (half) return launchFft2dLargeInverse(N, cplxView4(cplx), realView3(real), padL, padU, stream);
-  return FBFFT_UNSUPPORTED_SIZE;
+  return launchTwoPass(N, 3, cplx->data, cplx->stride[0], cplx->stride[1], cplx->stride[2],
+                       real->data, real->stride[0], real->stride[1], real->stride[2],
+                       real->size[0], real->size[1], real->size[2], padL, padU, stream);
 }
 
 }  // extern "C"
@@ -230,15 +234,32 @@ extern "C" int fbfft_conv_fprop(const fbfft_tensor* input, const fbfft_tensor* w
   return launchFft2dSmallInverse(N, spec(outSpec, B * Cout), out, 0, 0, stream);
 }
 
-// ---- entry points whose kernels are not wired yet ----
-extern "C" {
-int fbfft_c2c_2d_pass2(const fbfft_tensor*, const fbfft_tensor*, fbfft_stream_t) { return FBFFT_UNSUPPORTED_SIZE; }
-int fbfft_c2c_2d_inverse_pass1(const fbfft_tensor*, const fbfft_tensor*, fbfft_stream_t) { return FBFFT_UNSUPPORTED_SIZE; }
-int fbfft_iterated_conv(int fftSize, const fbfft_tile* ins, const fbfft_tile* outs,
-                        const fbfft_tensor* weight, int pass, float scale, int batchSize,
-                        size_t numTiles, fbfft_stream_t stream) {
-  if (!okTensor(weight, 4) || !ins || !outs) return 0;
-  return launchIteratedConv(fftSize, ins, outs, weight->data, weight->stride, weight->size, pass,
-                            scale, batchSize, numTiles, stream);
+extern "C" int fbfft_c2c_2d_pass2(const fbfft_tensor* src, const fbfft_tensor* dst,
+                                  fbfft_stream_t stream) {
+  if (!okTensor(src, 4) || !okTensor(dst, 4)) return FBFFT_UNSUPPORTED_DIMENSION;
+  const int N = src->size[1];
+  if (!(N == 64 || N == 128)) return FBFFT_UNSUPPORTED_SIZE;
+  if (src->size[2] != N / 2 + 1 || dst->size[1] != N / 2 + 1 || dst->size[2] != N)
+    return FBFFT_UNSUPPORTED_SIZE;
+  if (src->size[0] != dst->size[0] || src->data == dst->data) return FBFFT_UNSUPPORTED_DIMENSION;
+  if (!okCplx(src) || !okCplx(dst)) return FBFFT_UNSUPPORTED_DIMENSION;
+  if (empty(src)) return FBFFT_SUCCESS;
+  return launchTwoPass(N, 1, src->data, src->stride[0], src->stride[1], src->stride[2], dst->data,
+                       dst->stride[0], dst->stride[1], dst->stride[2], src->size[0], 0, 0, 0, 0,
+                       stream);
 }
+
+extern "C" int fbfft_c2c_2d_inverse_pass1(const fbfft_tensor* src, const fbfft_tensor* dst,
+                                          fbfft_stream_t stream) {
+  if (!okTensor(src, 4) || !okTensor(dst, 4)) return FBFFT_UNSUPPORTED_DIMENSION;
+  const int N = src->size[2];
+  // the size test of fbfft/FBIFFT2D-inl.cuh:537-542, narrowed to the sizes it dispatches
+  if (!(N == 64 || N == 128) || src->size[1] != N / 2 + 1) return FBFFT_UNSUPPORTED_SIZE;
+  if (dst->size[1] != N || dst->size[2] != N) return FBFFT_UNSUPPORTED_SIZE;
+  if (dst->size[0] < (src->size[0] + 1) / 2) return FBFFT_UNSUPPORTED_DIMENSION;
+  if (!okCplx(src) || !okCplx(dst)) return FBFFT_UNSUPPORTED_DIMENSION;
+  if (empty(src)) return FBFFT_SUCCESS;
+  return launchTwoPass(N, 2, src->data, src->stride[0], src->stride[1], src->stride[2], dst->data,
+                       dst->stride[0], dst->stride[1], dst->stride[2], src->size[0], 0, 0, 0, 0,
+                       stream);
 }

@@ -57,4 +57,8 @@ int launchIteratedConv(int N, const fbfft_tile* ins, const fbfft_tile* outs, flo
                        const int* wStride, const int* wSize, int pass, float scale, int batch,
                        size_t numTiles, hipStream_t s);
 
+// mode 0/1: forward pass 1/2, mode 2/3: inverse pass 1/2 of the two-call 64/128 forms
+int launchTwoPass(int N, int mode, float* src, long s0, long s1, long s2, float* dst, long d0,
+                  long d1, long d2, int B, int h, int w, int padL, int padU, hipStream_t s);
+
 }  // namespace fbfft_amd

@@ -1,0 +1,153 @@
+// The reference's two-call forms of the 64 x 64 and 128 x 128 transforms, kept
+// for callers that already own the scratch buffer and issue both calls
+// (forward: fbfft/FBFFT2D-inl.cuh:230-317 then :321-444; inverse:
+// fbfft/FBIFFT2D-inl.cuh:252-356 then :360-474).  New code should use the
+// single-kernel path in fft2d_large.hip, which produces the same result with one
+// pass over HBM.
+//
+// All four passes are batches of N-point complex FFTs that differ only in how a
+// transform's points are gathered and where its results go, so one kernel serves
+// them: a 256-lane workgroup stages 256/G transforms in LDS (G = N/32 lanes per
+// transform), runs the radix-G split + 32-point in-register FFT and scatters.
+#include "common.h"
+#include "fft_lds.h"
+#include "fft_regs.h"
+
+namespace fbfft_amd {
+namespace {
+
+constexpr int kTP = 256;
+
+struct TwoPassArgs {
+  float* src;      // real plane or complex-as-float
+  float* dst;
+  long s0, s1, s2;  // src strides (floats) of its three leading dims
+  long d0, d1, d2;  // dst strides (floats)
+  int B;            // planes (for the inverse: of the real / half-spectrum tensor)
+  int h, w, padL, padU;
+};
+
+// MODE 0: forward pass 1   real [B][h][w] window      -> scratch [B][N][N/2+1]   (rows)
+// MODE 1: forward pass 2   scratch [B][N][N/2+1]      -> dst [B][N/2+1][N]       (columns, transposed)
+// MODE 2: inverse pass 1   src [B][N/2+1][N]          -> scratch [ceil(B/2)][N][N], planes paired
+// MODE 3: inverse pass 2   scratch [ceil(B/2)][N][N]  -> real [B][h][w] window
+template <int N, int MODE>
+__global__ __launch_bounds__(kTP) void twoPassKernel(TwoPassArgs a, int total) {
+  constexpr int G = N / 32, L = 32, ROWS = kTP / G, RS = N + 1, nc = N / 2 + 1;
+  constexpr bool FWD = MODE < 2;
+  __shared__ __align__(8) c32 lds[ROWS * RS];
+  __shared__ __align__(8) c32 tw[256];
+  const int t = threadIdx.x;
+  const int q0 = blockIdx.x * ROWS;
+  const int half = (a.B + 1) / 2;
+  fillTwiddles<FWD>(tw, t, kTP);
+
+  auto cplxAt = [](const float* p) { return *reinterpret_cast<const float2*>(p); };
+  // Hermitian expansion of the half spectrum [N/2+1][N] (fbfft/FBIFFT2D-inl.cuh:61-97)
+  auto expand = [&](int b, int row, int col) {
+    const float* p = a.src + (long)b * a.s0;
+    if (row < nc) return cplxAt(p + (long)row * a.s1 + (long)col * a.s2);
+    c32 v = cplxAt(p + (long)(N - row) * a.s1 + (long)((N - col) % N) * a.s2);
+    return c32{v.x, -v.y};
+  };
+
+  for (int idx = t; idx < ROWS * N; idx += kTP) {
+    const int qi = idx / N, j = idx % N;
+    const int q = q0 + qi;
+    c32 v = c32{0.f, 0.f};
+    if (q < total) {
+      if (MODE == 0) {
+        const int b = q / N, y = q % N;
+        if (inWindow(y, j, a.padU, a.padL, a.h, a.w))
+          v.x = a.src[(long)b * a.s0 + (long)(y - a.padU) * a.s1 + (long)(j - a.padL) * a.s2];
+      } else if (MODE == 1) {
+        const int b = q / nc, kx = q % nc;
+        v = cplxAt(a.src + (long)b * a.s0 + (long)j * a.s1 + (long)kx * a.s2);
+      } else if (MODE == 2) {
+        const int b = q / N, row = q % N;
+        v = expand(b, row, j);
+        if (b + half < a.B) {
+          c32 u = expand(b + half, row, j);
+          v.x -= u.y;  // + i * u
+          v.y += u.x;
+        }
+      } else {
+        const int b = q / N, x = q % N;
+        v = cplxAt(a.src + (long)b * a.s0 + (long)j * a.s1 + (long)x * a.s2);
+      }
+    }
+    lds[qi * RS + j] = v;
+  }
+  __syncthreads();
+
+  const int row = t % ROWS, g = t / ROWS;
+  c32* z = lds + row * RS;
+  c32 v[L];
+  splitFFT<N, G, FWD>(z, g, tw, v);
+  __syncthreads();
+  staticFor<L>([&](auto kk) {
+    constexpr int k = decltype(kk)::value;
+    z[G * k + g] = v[slot<L>(k)];
+  });
+  __syncthreads();
+
+  for (int idx = t; idx < ROWS * N; idx += kTP) {
+    const int qi = idx / N, k = idx % N;
+    const int q = q0 + qi;
+    if (q >= total) break;
+    const c32 r = lds[qi * RS + k];
+    if (MODE == 0) {
+      const int b = q / N, y = q % N;
+      if (k < nc)
+        *reinterpret_cast<float2*>(a.dst + (long)b * a.d0 + (long)y * a.d1 + (long)k * a.d2) = r;
+    } else if (MODE == 1) {
+      const int b = q / nc, kx = q % nc;
+      *reinterpret_cast<float2*>(a.dst + (long)b * a.d0 + (long)kx * a.d1 + (long)k * a.d2) = r;
+    } else if (MODE == 2) {
+      const int b = q / N, rw = q % N;
+      *reinterpret_cast<float2*>(a.dst + (long)b * a.d0 + (long)rw * a.d1 + (long)k * a.d2) = r;
+    } else {
+      const int b = q / N, x = q % N;  // x: output row, k: output column
+      if (inWindow(x, k, a.padU, a.padL, a.h, a.w)) {
+        const long o = (long)(x - a.padU) * a.d1 + (long)(k - a.padL) * a.d2;
+        a.dst[(long)b * a.d0 + o] = r.x;
+        if (b + half < a.B) a.dst[(long)(b + half) * a.d0 + o] = r.y;
+      }
+    }
+  }
+}
+
+template <int N, int MODE>
+int launchMode(const TwoPassArgs& a, hipStream_t s) {
+  constexpr int ROWS = kTP / (N / 32), nc = N / 2 + 1;
+  const int half = (a.B + 1) / 2;
+  const int total = MODE == 0 ? a.B * N : MODE == 1 ? a.B * nc : half * N;
+  if (total <= 0) return FBFFT_SUCCESS;
+  twoPassKernel<N, MODE><<<dim3(ceilDiv(total, ROWS)), dim3(kTP), 0, s>>>(a, total);
+  return launchStatus();
+}
+
+}  // namespace
+
+int launchTwoPass(int N, int mode, float* src, long s0, long s1, long s2, float* dst, long d0,
+                  long d1, long d2, int B, int h, int w, int padL, int padU, hipStream_t s) {
+  TwoPassArgs a{src, dst, s0, s1, s2, d0, d1, d2, B, h, w, padL, padU};
+  if (N == 64) {
+    switch (mode) {
+      case 0: return launchMode<64, 0>(a, s);
+      case 1: return launchMode<64, 1>(a, s);
+      case 2: return launchMode<64, 2>(a, s);
+      case 3: return launchMode<64, 3>(a, s);
+    }
+  } else if (N == 128) {
+    switch (mode) {
+      case 0: return launchMode<128, 0>(a, s);
+      case 1: return launchMode<128, 1>(a, s);
+      case 2: return launchMode<128, 2>(a, s);
+      case 3: return launchMode<128, 3>(a, s);
+    }
+  }
+  return FBFFT_UNSUPPORTED_SIZE;
+}
+
+}  // namespace fbfft_amd

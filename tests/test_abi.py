@@ -79,3 +79,15 @@ def test_synth_is_deterministic():
     assert not bool((a == synth.normal((4, 8), seed=4)).all())
     u = synth.uniform((1000,), seed=0)
     assert float(u.min()) >= -1.0 and float(u.max()) < 1.0
+
+
+def test_cpp_facade_compiles_against_reference_include_paths():
+    """Host code that includes cuda/fbfft/FBFFT.cuh, cuda/MM.cuh and
+    cuda/fbfft/FFTIteratedConvolution.cuh and uses the reference's names builds and links."""
+    import subprocess
+    if not os.path.exists(F.LIB_PATH):
+        import __graft_entry__
+        __graft_entry__.build()
+    subprocess.check_call(["make", "-C", os.path.join(ROOT, "tests", "cpp"), "-B"],
+                          stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL)
+    assert os.path.exists(os.path.join(ROOT, "tests", "cpp", "facade_check"))
