@@ -263,3 +263,11 @@ extern "C" int fbfft_c2c_2d_inverse_pass1(const fbfft_tensor* src, const fbfft_t
                        dst->stride[0], dst->stride[1], dst->stride[2], src->size[0], 0, 0, 0, 0,
                        stream);
 }
+
+extern "C" int fbfft_iterated_conv(int fftSize, const fbfft_tile* ins, const fbfft_tile* outs,
+                                   const fbfft_tensor* weight, int pass, float scale,
+                                   int batchSize, size_t numTiles, fbfft_stream_t stream) {
+  if (!okTensor(weight, 4) || !ins || !outs) return 0;
+  return launchIteratedConv(fftSize, ins, outs, weight->data, weight->stride, weight->size, pass,
+                            scale, batchSize, numTiles, stream);
+}
