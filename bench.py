@@ -83,7 +83,7 @@ def cpu_baseline(x_host, N, budget_s=12.0):
     t0 = time.perf_counter()
     O.fbfft2d(x_host, N)
     one = time.perf_counter() - t0
-    reps = max(1, min(50, int(budget_s / max(one, 1e-3))))
+    reps = max(1, min(5000, int(budget_s / max(one, 1e-4))))
     t0 = time.perf_counter()
     for _ in range(reps):
         O.fbfft2d(x_host, N)
@@ -92,6 +92,71 @@ def cpu_baseline(x_host, N, budget_s=12.0):
     return {"value": round(gbs, 3), "unit": "GB/s", "cores": threads, "kind": "port",
             "sample": "%d passes of the full %d-plane %dx%d R2C batch, OpenMP over planes, "
                       "%.3f s per pass" % (reps, x_host.shape[0], N, N, dt)}
+
+
+def measured_traffic():
+    """HBM bytes per R2C launch from the committed rocprofv3 counter summary, or None."""
+    path = os.path.join(ROOT, "profiles", "fft2dSmallForward32_configs1.md")
+    try:
+        for line in open(path):
+            if line.startswith("traffic_bytes_per_launch:"):
+                return int(line.split(":")[1])
+    except OSError:
+        pass
+    return None
+
+
+def conv_extras(F, synth, torch, dev, extra):
+    """configs[3] FFT convolution forward (ms/iter) and its contraction; configs[4] tiled conv."""
+    x = synth.normal((128, 64, 27, 27), seed=30, device=dev)
+    w = synth.normal((192, 64, 5, 5), seed=31, std=0.02, device=dev)
+    out = torch.empty((128, 192, 23, 23), device=dev)
+    ws = torch.empty(F.conv_fprop_workspace(128, 64, 192, 32), dtype=torch.uint8, device=dev)
+    L = F.lib()
+    vx, vw, vo = F.view(x), F.view(w), F.view(out)
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    wsp, wsb = ctypes.c_void_p(ws.data_ptr()), ws.numel()
+
+    def conv():
+        rc = L.fbfft_conv_fprop(ctypes.byref(vx), ctypes.byref(vw), ctypes.byref(vo), 32, wsp, wsb,
+                                stream)
+        if rc != 0:
+            raise RuntimeError(F.error_string(rc))
+    _, t = timed(conv, 50, 5, torch)
+    extra["fft_conv_configs3_ms_per_iter"] = round(t * 1e3, 4)
+    extra["fft_conv_configs3_direct_equiv_TFLOPs"] = round(41.6e9 / t / 1e12, 1)
+    extra["fft_conv_configs3_fp32_peak_direct_ms"] = round(41.6e9 / 157.3e12 * 1e3, 4)
+    A = synth.normal((128, 64, 17, 32, 2), seed=30, device=dev)
+    Bm = synth.normal((192, 64, 17, 32, 2), seed=31, device=dev)
+    C = torch.empty((128, 192, 17, 32, 2), device=dev)
+    mm = prepared("fbfft_transpose_mm", F, A, Bm, C, 0, 1, 0, ctypes.c_float(1.0 / 1024))
+    _, t = timed(mm, 50, 5, torch)
+    extra["transposeMM_configs3_us"] = round(t * 1e6, 1)
+    extra["transposeMM_configs3_TFLOPs"] = round(6.845e9 / t / 1e12, 1)
+    extra["transposeMM_configs3_frac_of_fp32_mfma_peak"] = round(6.845e9 / t / 157.3e12, 4)
+    del A, Bm, C, x, w, out, ws
+    # configs[4]
+    x4 = synth.uniform((16, 32, 256, 256), seed=40, device=dev)
+    w4 = synth.normal((32, 32, 9, 9), seed=41, std=0.05, device=dev)
+    o4 = torch.empty((16, 32, 248, 248), device=dev)
+    iv, ov = [], []
+    for y0 in range(0, 248, 24):
+        for x0 in range(0, 248, 24):
+            iv.append((y0, x0, min(32, 256 - y0), min(32, 256 - x0), 0, 0))
+            ov.append((y0, x0, min(24, 248 - y0), min(24, 248 - x0), 0, 0))
+    ins, n = F.make_tiles(x4, iv)
+    outs, _ = F.make_tiles(o4, ov)
+    vw4 = F.view(w4)
+
+    def tiled():
+        rc = L.fbfft_iterated_conv(32, ctypes.c_void_p(ins.data_ptr()),
+                                   ctypes.c_void_p(outs.data_ptr()), ctypes.byref(vw4), 0,
+                                   ctypes.c_float(1.0), 16, n, stream)
+        if rc != 1:
+            raise RuntimeError("fbfft_iterated_conv returned %d" % rc)
+    _, t = timed(tiled, 10, 2, torch)
+    extra["iterated_conv_configs4_ms_per_iter"] = round(t * 1e3, 4)
+    extra["iterated_conv_configs4_direct_equiv_TFLOPs"] = round(163.3e9 / t / 1e12, 1)
 
 
 def main():
@@ -162,6 +227,7 @@ def main():
             extra["r2c_%dx%d_b%d_GBps" % (n2, n2, b2)] = round(nb / lf / 1e9, 1)
             extra["c2r_%dx%d_b%d_GBps" % (n2, n2, b2)] = round(nb / li / 1e9, 1)
             del x2, s2
+        conv_extras(F, synth, torch, dev, extra)
 
     out = {
         "metric": "fbfft2D 32x32 R2C GB/s (% HBM peak); FFT-conv ms/iter at configs[3]",
@@ -179,7 +245,7 @@ def main():
         "config": {"workload": "configs[1]: fbfft2D R2C, 16384 planes of 32x32 fp32 N(0,1) seed 1, "
                                "output [16384][17][32][2]; 8448 algorithmic bytes per plane"},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": measured_traffic(),
                      "kernel": "fft2dSmallForward<32>", "bytes_per_launch": nbytes,
                      "launch_us": round(launch_s * 1e6, 2)},
         "extra": extra,
