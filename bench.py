@@ -159,6 +159,54 @@ def conv_extras(F, synth, torch, dev, extra):
     extra["iterated_conv_configs4_direct_equiv_TFLOPs"] = round(163.3e9 / t / 1e12, 1)
 
 
+def run_only(name, steps, warmup, F, synth, torch, dev):
+    """One workload in a tight loop, for profiling."""
+    if name in ("r2c32", "c2r32", "r2c64", "c2r64", "r2c128", "c2r128"):
+        n = int(name[3:])
+        b = {32: 16384, 64: 16384, 128: 4096}[n]
+        x = synth.normal((b, n, n), seed=1, device=dev)
+        spec = torch.empty((b, n // 2 + 1, n, 2), device=dev)
+        fwd = prepared("fbfft_r2c_2d", F, x, spec, 0, 0)
+        fwd()
+        fn = fwd if name.startswith("r2c") else prepared("fbfft_c2r_2d", F, spec, x, 0, 0)
+        _, t = timed(fn, steps, warmup, torch)
+        return {"only": name, "us": round(t * 1e6, 2), "GBps": round(b * plane_bytes(n) / t / 1e9, 1)}
+    if name in ("r2c1d", "c2r1d"):
+        n, b = 256, 1 << 18
+        x = synth.uniform((b, n), seed=0, device=dev)
+        spec = torch.empty((b, n // 2 + 1, 2), device=dev)
+        fwd = prepared("fbfft_r2c_1d", F, x, spec, 0)
+        fwd()
+        fn = fwd if name == "r2c1d" else prepared("fbfft_c2r_1d", F, x, spec, 0)
+        _, t = timed(fn, steps, warmup, torch)
+        return {"only": name, "us": round(t * 1e6, 2),
+                "GBps": round(b * (4 * n + 8 * (n // 2 + 1)) / t / 1e9, 1)}
+    extra = {}
+    if name == "mm":
+        A = synth.normal((128, 64, 17, 32, 2), seed=30, device=dev)
+        Bm = synth.normal((192, 64, 17, 32, 2), seed=31, device=dev)
+        C = torch.empty((128, 192, 17, 32, 2), device=dev)
+        mm = prepared("fbfft_transpose_mm", F, A, Bm, C, 0, 1, 0, ctypes.c_float(1.0 / 1024))
+        _, t = timed(mm, steps, warmup, torch)
+        return {"only": name, "us": round(t * 1e6, 2), "TFLOPs": round(6.845e9 / t / 1e12, 2)}
+    if name == "conv":
+        x = synth.normal((128, 64, 27, 27), seed=30, device=dev)
+        w = synth.normal((192, 64, 5, 5), seed=31, std=0.02, device=dev)
+        out = torch.empty((128, 192, 23, 23), device=dev)
+        ws = torch.empty(F.conv_fprop_workspace(128, 64, 192, 32), dtype=torch.uint8, device=dev)
+        stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+        vx, vw, vo = F.view(x), F.view(w), F.view(out)
+
+        def conv():
+            rc = F.lib().fbfft_conv_fprop(ctypes.byref(vx), ctypes.byref(vw), ctypes.byref(vo), 32,
+                                          ctypes.c_void_p(ws.data_ptr()), ws.numel(), stream)
+            assert rc == 0
+        _, t = timed(conv, steps, warmup, torch)
+        return {"only": name, "us": round(t * 1e6, 2)}
+    conv_extras(F, synth, torch, dev, extra)
+    return {"only": name, **extra}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -166,6 +214,10 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the informative extra configs")
+    ap.add_argument("--only", default=None,
+                    choices=["r2c32", "c2r32", "r2c64", "c2r64", "r2c128", "c2r128", "mm", "conv",
+                             "iterconv", "r2c1d", "c2r1d"],
+                    help="run just this workload --steps times (for rocprofv3) and print its timing")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="only run a plain 256 MiB device-to-device copy 20 times: the known-size "
                          "kernel that FETCH_SIZE / WRITE_SIZE counter readings are scaled by")
@@ -192,6 +244,10 @@ def main():
         torch.cuda.synchronize()
         print(json.dumps({"calibrate_copy_bytes_read": a.numel() * 4,
                           "calibrate_copy_bytes_written": a.numel() * 4, "launches": 20}))
+        return
+
+    if args.only:
+        print(json.dumps(run_only(args.only, args.steps, args.warmup, F, synth, torch, dev)))
         return
 
     N, B = 32, 16384

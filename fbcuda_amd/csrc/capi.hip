@@ -173,23 +173,10 @@ extern "C" int fbfft_transpose_mm(const fbfft_tensor* A, const fbfft_tensor* B,
                            conjA != 0, conjB != 0, accumulate != 0, invNorm, stream);
 }
 
-namespace {
-size_t specFloats(int planes, int N) { return (size_t)planes * (N / 2 + 1) * N * 2; }
-
-// [d0][d1][h][w] -> [d0*d1][h][w] when the two leading dimensions collapse
-bool collapse4(const fbfft_tensor* t, RealView* v) {
-  if (t->size[0] > 1 && t->stride[0] != (long)t->stride[1] * t->size[1]) return false;
-  *v = RealView{t->data, t->stride[1], t->stride[2], t->stride[3],
-                t->size[0] * t->size[1], t->size[2], t->size[3]};
-  return true;
-}
-}  // namespace
-
 extern "C" size_t fbfft_conv_fprop_workspace(int batch, int cin, int cout, int fftSize) {
   if (batch <= 0 || cin <= 0 || cout <= 0) return 0;
-  const size_t fl = specFloats(batch * cin, fftSize) + specFloats(cout * cin, fftSize) +
-                    specFloats(batch * cout, fftSize);
-  return fl * sizeof(float);
+  if (!(fftSize == 8 || fftSize == 16 || fftSize == 32)) return 0;
+  return convFpropWorkspaceBytes(fftSize, batch, cin, cout);
 }
 
 extern "C" int fbfft_conv_fprop(const fbfft_tensor* input, const fbfft_tensor* weight,
@@ -210,28 +197,9 @@ extern "C" int fbfft_conv_fprop(const fbfft_tensor* input, const fbfft_tensor* w
   if (!workspace || !aligned(workspace, 256) ||
       workspaceBytes < fbfft_conv_fprop_workspace(B, Cin, Cout, N))
     return FBFFT_UNSUPPORTED_DIMENSION;
-  RealView in, wt, out;
-  if (!collapse4(input, &in) || !collapse4(weight, &wt) || !collapse4(output, &out))
-    return FBFFT_UNSUPPORTED_DIMENSION;
-
-  const int rows = N / 2 + 1;
-  const int plane = rows * N * 2;  // floats per spectrum plane
-  float* inSpec = static_cast<float*>(workspace);
-  float* wtSpec = inSpec + specFloats(B * Cin, N);
-  float* outSpec = wtSpec + specFloats(Cout * Cin, N);
-  auto spec = [&](float* p, int planes) { return CplxView{p, plane, 2 * N, 2, planes, rows, N}; };
-
-  int rc = launchFft2dSmallForward(N, in, spec(inSpec, B * Cin), 0, 0, stream);
-  if (rc != FBFFT_SUCCESS) return rc;
-  rc = launchFft2dSmallForward(N, wt, spec(wtSpec, Cout * Cin), 0, 0, stream);
-  if (rc != FBFFT_SUCCESS) return rc;
-  // o(b, f) = sum_p i(b, p) . conj(w(f, p)), scaled by 1/N^2 (MM-inl.cuh:193-196)
-  rc = launchTransposeMM(inSpec, (long)Cin * plane, plane, wtSpec, (long)Cin * plane, plane,
-                         outSpec, (long)Cout * plane, plane, B, Cout, Cin, rows * N, false, true,
-                         false, 1.0f / (float)(N * N), stream);
-  if (rc != FBFFT_SUCCESS) return rc;
-  // the valid region is the top-left corner of the inverse transform: crop on store
-  return launchFft2dSmallInverse(N, spec(outSpec, B * Cout), out, 0, 0, stream);
+  return launchConvFprop(N, input->data, input->stride, input->size, weight->data, weight->stride,
+                         weight->size, output->data, output->stride, output->size, workspace,
+                         stream);
 }
 
 extern "C" int fbfft_c2c_2d_pass2(const fbfft_tensor* src, const fbfft_tensor* dst,

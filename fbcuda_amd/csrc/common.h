@@ -61,4 +61,9 @@ int launchIteratedConv(int N, const fbfft_tile* ins, const fbfft_tile* outs, flo
 int launchTwoPass(int N, int mode, float* src, long s0, long s1, long s2, float* dst, long d0,
                   long d1, long d2, int B, int h, int w, int padL, int padU, hipStream_t s);
 
+size_t convFpropWorkspaceBytes(int N, int B, int Cin, int Cout);
+int launchConvFprop(int N, float* in, const int* inStride, const int* inSize, float* wt,
+                    const int* wtStride, const int* wtSize, float* out, const int* outStride,
+                    const int* outSize, void* workspace, hipStream_t s);
+
 }  // namespace fbfft_amd
