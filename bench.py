@@ -190,10 +190,11 @@ def run_only(name, steps, warmup, F, synth, torch, dev):
         _, t = timed(mm, steps, warmup, torch)
         return {"only": name, "us": round(t * 1e6, 2), "TFLOPs": round(6.845e9 / t / 1e12, 2)}
     if name == "conv":
-        x = synth.normal((128, 64, 27, 27), seed=30, device=dev)
+        nb = int(os.environ.get("FBFFT_BENCH_CONV_B", "128"))  # profiling aid: other batch sizes
+        x = synth.normal((nb, 64, 27, 27), seed=30, device=dev)
         w = synth.normal((192, 64, 5, 5), seed=31, std=0.02, device=dev)
-        out = torch.empty((128, 192, 23, 23), device=dev)
-        ws = torch.empty(F.conv_fprop_workspace(128, 64, 192, 32), dtype=torch.uint8, device=dev)
+        out = torch.empty((nb, 192, 23, 23), device=dev)
+        ws = torch.empty(F.conv_fprop_workspace(nb, 64, 192, 32), dtype=torch.uint8, device=dev)
         stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
         vx, vw, vo = F.view(x), F.view(w), F.view(out)
 

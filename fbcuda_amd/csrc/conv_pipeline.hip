@@ -20,6 +20,8 @@
 //      consecutive j per bin, inverse transform, crop on store.
 //
 // Spectra are unpacked (N/2+1 rows) so the contraction is a plain complex GEMM.
+#include <stdlib.h>
+
 #include "common.h"
 #include "fft2d_core.h"
 #include "fft_regs.h"
@@ -106,14 +108,22 @@ __global__ __launch_bounds__(kT) void inverseBinMajor(const float2* Cs, int I, i
 
   const int sp = t % SLOTS, bq = t / SLOTS;
   {
+    // gather: every load is issued before the first LDS store
+    constexpr int PER = C::BINS / T;
+    static_assert(C::BINS % T == 0, "bins divide evenly over the lane groups");
     c32* dstp = lds + sp * PSZ;
     const float2* src = Cs + (long)i * Jp + j0 + sp;
     const long binStride = (long)I * Jp;
-#pragma unroll 2
-    for (int bin = bq; bin < C::BINS; bin += T) {
-      const int r = bin / N, x = bin % N;
-      dstp[r * RS + x] = src[bin * binStride];
-    }
+    c32 in[PER];
+    staticFor<PER>([&](auto uu) {
+      constexpr int u = decltype(uu)::value;
+      in[u] = src[(bq + T * u) * binStride];
+    });
+    staticFor<PER>([&](auto uu) {
+      constexpr int u = decltype(uu)::value;
+      const int bin = bq + T * u;
+      dstp[(bin / N) * RS + bin % N] = in[u];
+    });
   }
   __syncthreads();
   c32* plane = lds + s * PSZ;
@@ -141,7 +151,7 @@ __global__ __launch_bounds__(kT) void inverseBinMajor(const float2* Cs, int I, i
 }
 
 // ---- 2. batched complex GEMM, bin-major ----
-constexpr int GI = 128, GJ = 64, GK = 8;
+constexpr int GI = 128;
 
 struct GemmArgs {
   const float2* A;  // [bins][Kp][Ip]
@@ -152,7 +162,11 @@ struct GemmArgs {
   float invNorm;
 };
 
+template <int GJ, int GK>
 __global__ __launch_bounds__(kT, 2) void binGemm(GemmArgs g) {
+  constexpr int NA = GK * GI / 2 / kT;                 // float4 of A per lane per slice
+  constexpr int NB = (GK * GJ / 2 + kT - 1) / kT;      // float4 of B per lane per slice
+  constexpr int NQ = GJ / 32;  // 32-column MFMA sub-tiles per wave
   __shared__ __align__(16) float2 As[2][GK][GI];
   __shared__ __align__(16) float2 Bs[2][GK][GJ];
   const int t = threadIdx.x;
@@ -171,9 +185,9 @@ __global__ __launch_bounds__(kT, 2) void binGemm(GemmArgs g) {
   const float2* Ab = g.A + (long)bin * g.Kp * g.Ip;
   const float2* Bb = g.B + (long)bin * g.Kp * g.Jp;
 
-  floatx16 cre[2], cim[2];
+  floatx16 cre[NQ], cim[NQ];
 #pragma unroll
-  for (int q = 0; q < 2; ++q)
+  for (int q = 0; q < NQ; ++q)
 #pragma unroll
     for (int v = 0; v < 16; ++v) {
       cre[q][v] = 0.f;
@@ -181,28 +195,37 @@ __global__ __launch_bounds__(kT, 2) void binGemm(GemmArgs g) {
     }
 
   // slice loads: A 8 x 128 complex = 512 float4 (2 per lane), B 8 x 64 = 256 float4 (1 per lane)
-  float4 ra[2], rb;
+  float4 ra[NA], rb[NB];
   auto fetch = [&](int k0) {
 #pragma unroll
-    for (int u = 0; u < 2; ++u) {
+    for (int u = 0; u < NA; ++u) {
       const int idx = t + kT * u;
       const int kk = idx / (GI / 2), ii = 2 * (idx % (GI / 2));
       ra[u] = float4{0.f, 0.f, 0.f, 0.f};
       if (k0 + kk < g.Kp && i0 + ii < g.Ip)
         ra[u] = *reinterpret_cast<const float4*>(Ab + (long)(k0 + kk) * g.Ip + i0 + ii);
     }
-    const int kk = t / (GJ / 2), jj = 2 * (t % (GJ / 2));
-    rb = float4{0.f, 0.f, 0.f, 0.f};
-    if (k0 + kk < g.Kp && j0 + jj < g.Jp)
-      rb = *reinterpret_cast<const float4*>(Bb + (long)(k0 + kk) * g.Jp + j0 + jj);
+#pragma unroll
+    for (int u = 0; u < NB; ++u) {
+      const int idx = t + kT * u;
+      const int kk = idx / (GJ / 2), jj = 2 * (idx % (GJ / 2));
+      rb[u] = float4{0.f, 0.f, 0.f, 0.f};
+      if (kk < GK && k0 + kk < g.Kp && j0 + jj < g.Jp)
+        rb[u] = *reinterpret_cast<const float4*>(Bb + (long)(k0 + kk) * g.Jp + j0 + jj);
+    }
   };
   auto stash = [&](int buf) {
 #pragma unroll
-    for (int u = 0; u < 2; ++u) {
+    for (int u = 0; u < NA; ++u) {
       const int idx = t + kT * u;
       *reinterpret_cast<float4*>(&As[buf][idx / (GI / 2)][2 * (idx % (GI / 2))]) = ra[u];
     }
-    *reinterpret_cast<float4*>(&Bs[buf][t / (GJ / 2)][2 * (t % (GJ / 2))]) = rb;
+#pragma unroll
+    for (int u = 0; u < NB; ++u) {
+      const int idx = t + kT * u;
+      if (idx / (GJ / 2) < GK)
+        *reinterpret_cast<float4*>(&Bs[buf][idx / (GJ / 2)][2 * (idx % (GJ / 2))]) = rb[u];
+    }
   };
 
   fetch(0);
@@ -217,7 +240,7 @@ __global__ __launch_bounds__(kT, 2) void binGemm(GemmArgs g) {
       const float2 a = As[cur][2 * s2 + h][32 * w + r];
       const float nar = -a.x;
 #pragma unroll
-      for (int q = 0; q < 2; ++q) {
+      for (int q = 0; q < NQ; ++q) {
         const float2 b = Bs[cur][2 * s2 + h][32 * q + r];
         // a * conj(b): re = ar*br + ai*bi, im = ai*br - ar*bi
         cre[q] = __builtin_amdgcn_mfma_f32_32x32x2f32(a.x, b.x, cre[q], 0, 0, 0);
@@ -233,7 +256,7 @@ __global__ __launch_bounds__(kT, 2) void binGemm(GemmArgs g) {
   // register v of lane (r, h) holds row 8*(v/4) + 4*h + v%4 and column r of a sub-tile
   float2* Cb = g.C + (long)bin * g.I * g.Jp;
 #pragma unroll
-  for (int q = 0; q < 2; ++q) {
+  for (int q = 0; q < NQ; ++q) {
     const int j = j0 + 32 * q + r;
     if (j >= g.Jp) continue;
 #pragma unroll
@@ -275,10 +298,16 @@ int runFprop(const PlaneSet& in, const PlaneSet& wt, const PlaneSet& out, int B,
   g.Jp = Jp;
   g.Kp = Kp;
   g.IT = ceilDiv(B, GI);
-  g.JT = ceilDiv(Jp, GJ);
   g.invNorm = 1.0f / (float)(N * N);
-  const int total = bins * g.IT * g.JT;
-  binGemm<<<dim3(roundUp(total, 8)), dim3(kT), 0, s>>>(g);
+  static const int gjEnv = getenv("FBFFT_GEMM_GJ") ? atoi(getenv("FBFFT_GEMM_GJ")) : 64;
+  static const int gkEnv = getenv("FBFFT_GEMM_GK") ? atoi(getenv("FBFFT_GEMM_GK")) : 8;
+  g.JT = ceilDiv(Jp, gjEnv == 32 ? 32 : 64);
+  const dim3 grid(roundUp(bins * g.IT * g.JT, 8));
+  if (gjEnv == 32 && gkEnv == 16) binGemm<32, 16><<<grid, dim3(kT), 0, s>>>(g);
+  else if (gjEnv == 32) binGemm<32, 8><<<grid, dim3(kT), 0, s>>>(g);
+  else if (gkEnv == 16) binGemm<64, 16><<<grid, dim3(kT), 0, s>>>(g);
+  else if (gkEnv == 4) binGemm<64, 4><<<grid, dim3(kT), 0, s>>>(g);
+  else binGemm<64, 8><<<grid, dim3(kT), 0, s>>>(g);
   inverseBinMajor<N><<<dim3(Jp / SL, B), dim3(kT), 0, s>>>(SC, B, Jp, out);
   return launchStatus();
 }

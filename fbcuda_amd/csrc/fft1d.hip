@@ -50,24 +50,30 @@ __global__ __launch_bounds__(k1dThreads) void fft1dForward(Row1D a) {
   const int b0 = blockIdx.x * ROWS;
   fillTwiddles<true>(tw, t, k1dThreads);
 
-  // ---- rows -> LDS as packed complex z[j] = (x[2j], x[2j+1]) ----
-  for (int idx = t; idx < ROWS * H; idx += k1dThreads) {
-    const int row = idx / H, j = idx % H;
-    const int b = b0 + row;
-    c32 v = c32{0.0f, 0.0f};
-    if (b < a.B) {
-      if constexpr (FAST) {
-        v = *reinterpret_cast<const float2*>(a.real + (size_t)b * a.sb + 2 * j);
-      } else {
-        const float* src = a.real + (size_t)b * a.sb;
-        const int x0 = 2 * j - a.padL, x1 = 2 * j + 1 - a.padL;
-        // a right shift that drops the last padL samples (fbfft/FBFFTCommon.cuh:325)
-        if (x0 >= 0) v.x = src[(size_t)x0 * a.sx];
-        if (x1 >= 0) v.y = src[(size_t)x1 * a.sx];
-      }
+  // ---- rows -> LDS as packed complex z[j] = (x[2j], x[2j+1]); every load is
+  // issued before the first one is consumed ----
+  constexpr int LOADS = (ROWS * H + k1dThreads - 1) / k1dThreads;
+  c32 in[LOADS];
+  staticFor<LOADS>([&](auto ii) {
+    constexpr int i = decltype(ii)::value;
+    const int idx = t + k1dThreads * i;
+    const int row = min(idx / H, ROWS - 1), j = idx % H;
+    const int b = min(b0 + row, a.B - 1);
+    if constexpr (FAST) {
+      in[i] = *reinterpret_cast<const float2*>(a.real + (size_t)b * a.sb + 2 * j);
+    } else {
+      const float* src = a.real + (size_t)b * a.sb;
+      const int x0 = 2 * j - a.padL, x1 = 2 * j + 1 - a.padL;
+      // a right shift that drops the last padL samples (fbfft/FBFFTCommon.cuh:325)
+      in[i].x = x0 >= 0 ? src[(size_t)x0 * a.sx] : 0.0f;
+      in[i].y = x1 >= 0 ? src[(size_t)x1 * a.sx] : 0.0f;
     }
-    lds[row * RS + j] = v;
-  }
+  });
+  staticFor<LOADS>([&](auto ii) {
+    constexpr int i = decltype(ii)::value;
+    const int idx = t + k1dThreads * i;
+    if (idx < ROWS * H) lds[(idx / H) * RS + idx % H] = in[i];
+  });
   __syncthreads();
 
   const int row = t % ROWS, g = t / ROWS;
@@ -113,13 +119,21 @@ __global__ __launch_bounds__(k1dThreads) void fft1dInverse(Row1D a) {
   const int b0 = blockIdx.x * ROWS;
   fillTwiddles<false>(tw, t, k1dThreads);
 
-  // ---- spectra -> LDS ----
-  for (int idx = t; idx < ROWS * (H + 1); idx += k1dThreads) {
-    const int r = idx / (H + 1), k = idx % (H + 1);
+  // ---- spectra -> LDS, all loads in flight together ----
+  constexpr int LOADS = (ROWS * (H + 1) + k1dThreads - 1) / k1dThreads;
+  c32 in[LOADS];
+  staticFor<LOADS>([&](auto ii) {
+    constexpr int i = decltype(ii)::value;
+    const int idx = t + k1dThreads * i;
+    const int r = min(idx / (H + 1), ROWS - 1), k = idx % (H + 1);
     const int b = min(b0 + r, a.B - 1);
-    lds[r * RS + k] =
-        *reinterpret_cast<const float2*>(a.cplx + (size_t)b * a.cb + (size_t)k * a.ck);
-  }
+    in[i] = *reinterpret_cast<const float2*>(a.cplx + (size_t)b * a.cb + (size_t)k * a.ck);
+  });
+  staticFor<LOADS>([&](auto ii) {
+    constexpr int i = decltype(ii)::value;
+    const int idx = t + k1dThreads * i;
+    if (idx < ROWS * (H + 1)) lds[(idx / (H + 1)) * RS + idx % (H + 1)] = in[i];
+  });
   __syncthreads();
 
   // ---- inverse real fix-up in place: bins k and H-k form one work item ----

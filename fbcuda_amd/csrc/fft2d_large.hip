@@ -159,44 +159,40 @@ __global__ __launch_bounds__(LargeCfg<N>::THREADS) void fft2dLargeInverse(CplxVi
   fillTwiddles<false>(tw, t, THREADS);
   c32* cb = reinterpret_cast<c32*>(buf);
 
-  // ---- copy in [kx][ky]; row H is folded into row 0: Z = F0 + i*FH ----
-  constexpr int ITERS = (C::F4_CPLX + THREADS - 1) / THREADS;
-  // rows 0..H-1 first, then row H is added into row 0 after a barrier
+  // ---- copy in [kx][ky].  All loads are issued before any is consumed (no load
+  // sits behind a branch or a barrier); the lanes that hold row 0 also fetch row H
+  // and store the fold Z = F0 + i*FH. ----
+  static_assert(H * (N / 2) % THREADS == 0, "rows 0..H-1 divide evenly over the lanes");
+  constexpr int ITERS = H * (N / 2) / THREADS;
+  auto fetch4 = [&](int r, int ky, int q) {
+    if constexpr (FAST_CPLX) {
+      return reinterpret_cast<const float4*>(cplx.data + (size_t)b * cplx.sb)[q];
+    } else {
+      const float* src = cplx.data + (size_t)b * cplx.sb + (size_t)r * cplx.sr + (size_t)ky * cplx.sc;
+      float2 a = *reinterpret_cast<const float2*>(src);
+      float2 c = *reinterpret_cast<const float2*>(src + cplx.sc);
+      return float4{a.x, a.y, c.x, c.y};
+    }
+  };
+  float4 in[ITERS];
   staticFor<ITERS>([&](auto ii) {
     constexpr int i = decltype(ii)::value;
     const int q = t + THREADS * i;
-    if (q < H * (N / 2)) {
-      const int r = q / (N / 2);
-      const int ky = 2 * (q % (N / 2));
-      float4 v;
-      if constexpr (FAST_CPLX) {
-        v = reinterpret_cast<const float4*>(cplx.data + (size_t)b * cplx.sb)[q];
-      } else {
-        const float* src = cplx.data + (size_t)b * cplx.sb + (size_t)r * cplx.sr + (size_t)ky * cplx.sc;
-        float2 a = *reinterpret_cast<const float2*>(src);
-        float2 c = *reinterpret_cast<const float2*>(src + cplx.sc);
-        v = float4{a.x, a.y, c.x, c.y};
-      }
-      cb[r * CS + ky] = c32{v.x, v.y};
-      cb[r * CS + ky + 1] = c32{v.z, v.w};
-    }
+    in[i] = fetch4(q / (N / 2), 2 * (q % (N / 2)), q);
   });
-  __syncthreads();
-  if (t < N / 2) {
-    const int ky = 2 * t;
-    float4 v;
-    if constexpr (FAST_CPLX) {
-      v = reinterpret_cast<const float4*>(cplx.data + (size_t)b * cplx.sb)[H * (N / 2) + t];
-    } else {
-      const float* src = cplx.data + (size_t)b * cplx.sb + (size_t)H * cplx.sr + (size_t)ky * cplx.sc;
-      float2 a = *reinterpret_cast<const float2*>(src);
-      float2 c = *reinterpret_cast<const float2*>(src + cplx.sc);
-      v = float4{a.x, a.y, c.x, c.y};
-    }
-    c32 a0 = cb[ky], a1 = cb[ky + 1];
-    cb[ky] = c32{a0.x - v.y, a0.y + v.x};
-    cb[ky + 1] = c32{a1.x - v.w, a1.y + v.z};
+  {
+    const int tq = t % (N / 2);  // lanes beyond the first N/2 fetch a duplicate they ignore
+    const float4 u = fetch4(H, 2 * tq, H * (N / 2) + tq);
+    if (t < N / 2) in[0] = float4{in[0].x - u.y, in[0].y + u.x, in[0].z - u.w, in[0].w + u.z};
   }
+  staticFor<ITERS>([&](auto ii) {
+    constexpr int i = decltype(ii)::value;
+    const int q = t + THREADS * i;
+    const int r = q / (N / 2);
+    const int ky = 2 * (q % (N / 2));
+    cb[r * CS + ky] = c32{in[i].x, in[i].y};
+    cb[r * CS + ky + 1] = c32{in[i].z, in[i].w};
+  });
   __syncthreads();
 
   // ---- column pass (inverse) ----
