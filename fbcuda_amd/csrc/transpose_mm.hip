@@ -27,6 +27,8 @@ typedef float floatx16 __attribute__((ext_vector_type(16)));
 constexpr int TI = 32, TJ = 32, XB = 16, KC = 4, THREADS = 256;  // 4 waves
 constexpr int XS = KC * 32 + 4;              // bin stride of an LDS plane (dwords), padded
 constexpr int PLANE = XB * XS;               // one of Ar, Ai, Br, Bi
+constexpr int CSTR = XB + 1;                 // padded bin stride of the C staging buffer (complex)
+constexpr int LDS_FLOATS = (4 * PLANE > 8 * 32 * CSTR * 2) ? 4 * PLANE : 8 * 32 * CSTR * 2;
 
 struct MMArgs {
   const float* A;
@@ -40,6 +42,7 @@ struct MMArgs {
   float aSign, bSign;  // -1 when the operand is conjugated
   float invNorm;
   int accumulate;
+  int chunks;  // ceil(XY / XB)
 };
 
 // 16 bins x 4 k x 32 rows of one operand: each lane fetches two float4 (bins
@@ -102,7 +105,7 @@ __device__ __forceinline__ void stashSlice(float* re, float* im, const Fetch& f,
 
 template <bool VEC4>
 __global__ __launch_bounds__(THREADS, 2) void transposeMMKernel(MMArgs a) {
-  __shared__ float lds[4 * PLANE];
+  __shared__ __align__(8) float lds[LDS_FLOATS];
   float* Ar = lds;
   float* Ai = lds + PLANE;
   float* Br = lds + 2 * PLANE;
@@ -110,9 +113,18 @@ __global__ __launch_bounds__(THREADS, 2) void transposeMMKernel(MMArgs a) {
 
   const int t = threadIdx.x;
   const int lane = t % 64, w = t / 64;
-  const int x0 = blockIdx.x * XB;
-  const int j0 = blockIdx.y * TJ;
-  const int i0 = blockIdx.z * TI;
+  // Workgroups are dealt round-robin to the 8 XCDs, each with its own L2.  Give
+  // every XCD a contiguous range of logical ids, ordered bin-chunk first, so that
+  // all (i, j) tiles that re-read the same lines of A and B share one L2.
+  const int tilesJ = (a.J + TJ - 1) / TJ, tilesI = (a.I + TI - 1) / TI;
+  const int total = a.chunks * tilesI * tilesJ;
+  const int per = (total + 7) / 8;
+  const int logical = (blockIdx.x % 8) * per + blockIdx.x / 8;
+  if (logical >= total) return;
+  const int x0 = (logical / (tilesI * tilesJ)) * XB;
+  const int rem = logical % (tilesI * tilesJ);
+  const int j0 = (rem % tilesJ) * TJ;
+  const int i0 = (rem / tilesJ) * TI;
 
   floatx16 cre[4], cim[4];
 #pragma unroll
@@ -156,27 +168,40 @@ __global__ __launch_bounds__(THREADS, 2) void transposeMMKernel(MMArgs a) {
     }
   }
 
-  // accumulator layout of the 32x32 tile: register r of lane l holds
-  // row 8*(r/4) + 4*(l/32) + r%4, column l%32
-  const int j = j0 + lane % 32;
-  const int xb = x0 + 4 * w;
-  if (j < a.J && xb < a.XY) {
+  // ---- epilogue: C leaves through LDS so that every store covers whole 128-byte
+  // runs (the 16 bins of one (i, j) element); written straight from the
+  // accumulators each lane would scatter 8-byte pieces 4 KB apart.
+  // Register r of lane l holds row 8*(r/4) + 4*(l/32) + r%4, column l%32, so the
+  // four registers 4c..4c+3 of all lanes form rows 8c..8c+7: one chunk.
+  float2* stage = reinterpret_cast<float2*>(lds);  // [8 rows][32 cols][CSTR] complex
+  const int col = lane % 32, hh = lane / 32;
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const int i = i0 + 8 * (r / 4) + 4 * (lane / 32) + r % 4;
-      if (i >= a.I) continue;
-      float* dst = a.C + (long)i * a.cRow + (long)j * a.cCol + 2L * xb;
+  for (int c = 0; c < 4; ++c) {
+    __syncthreads();  // operand slices / previous chunk fully consumed
 #pragma unroll
-      for (int b = 0; b < 4; ++b) {
-        if (xb + b < a.XY) {
-          float2 acc = float2{cre[b][r], cim[b][r]};
-          if (a.accumulate) {
-            float2 old = *reinterpret_cast<const float2*>(dst + 2 * b);
-            acc.x += old.x;
-            acc.y += old.y;
-          }
-          *reinterpret_cast<float2*>(dst + 2 * b) = float2{acc.x * a.invNorm, acc.y * a.invNorm};
+    for (int rr = 0; rr < 4; ++rr) {
+      const int row = 4 * hh + rr;
+#pragma unroll
+      for (int b = 0; b < 4; ++b)
+        stage[(row * 32 + col) * CSTR + 4 * w + b] = float2{cre[b][4 * c + rr], cim[b][4 * c + rr]};
+    }
+    __syncthreads();
+    // 256 (row, col) elements x 16 bins: 16 lanes per element, 16 elements per pass
+    const int xl = t % 16;
+#pragma unroll
+    for (int pass = 0; pass < 16; ++pass) {
+      const int e = t / 16 + 16 * pass;  // 0..255
+      const int row = e / 32, cc = e % 32;
+      const int i = i0 + 8 * c + row, j = j0 + cc, x = x0 + xl;
+      if (i < a.I && j < a.J && x < a.XY) {
+        float2 acc = stage[(row * 32 + cc) * CSTR + xl];
+        float* dst = a.C + (long)i * a.cRow + (long)j * a.cCol + 2L * x;
+        if (a.accumulate) {
+          float2 old = *reinterpret_cast<const float2*>(dst);
+          acc.x += old.x;
+          acc.y += old.y;
         }
+        *reinterpret_cast<float2*>(dst) = float2{acc.x * a.invNorm, acc.y * a.invNorm};
       }
     }
   }
@@ -209,7 +234,9 @@ int launchTransposeMM(const float* A, long a0, long a1, const float* B, long b0,
   m.bSign = conjB ? -1.f : 1.f;
   m.invNorm = invNorm;
   m.accumulate = accumulate ? 1 : 0;
-  dim3 grid(ceilDiv(XY, XB), ceilDiv(J, TJ), ceilDiv(I, TI)), block(THREADS);
+  m.chunks = ceilDiv(XY, XB);
+  const int total = m.chunks * ceilDiv(J, TJ) * ceilDiv(I, TI);
+  dim3 grid((total + 7) / 8 * 8), block(THREADS);
   const bool vec4 = aligned(A, 16) && aligned(B, 16) && a0 % 4 == 0 && a1 % 4 == 0 &&
                     b0 % 4 == 0 && b1 % 4 == 0;
   if (vec4)
