@@ -6,17 +6,20 @@
 //
 // Operands keep the reference layout: complex, xy innermost and contiguous, so
 // xy is the batch index of 'XY' independent small GEMMs and a coalesced global
-// access is a run of consecutive bins of one (row, col) element.
+// access is a run of consecutive bins of one (row, col) element.  Accumulators
+// are needed for every bin of a run at once, which bounds the tile: a workgroup
+// of 8 waves owns a 64 x 64 tile of C for 8 consecutive bins (64-byte runs; the
+// other half of each line goes to the neighbouring workgroup on the same XCD),
+// wave w owning bin w: 4 MFMA 32x32 sub-tiles x (re, im) = 128 accumulator
+// registers per lane.
 //
-// A workgroup (4 waves) owns a 32 x 32 tile of C for 16 consecutive bins (one
-// 128-byte line per element).  Per 4-deep slice of k it stages opA and opB in
-// LDS split into real and imaginary planes [bin][k][row], conjugation folded
-// into the sign of the imaginary plane, while the next slice is already in
-// flight in registers.  Wave w then runs bins 4w..4w+3 with
-// v_mfma_f32_32x32x2_f32: four real products per complex product,
-//   Cre += Ar*Br + (-Ai)*Bi,   Cim += Ar*Bi + Ai*Br,
-// 128 accumulator registers per lane.  Only this contraction uses MFMA; it is
-// the one dense product of the convolution path.
+// Per 4-deep slice of k the workgroup stages opA and opB in LDS split into real
+// and imaginary planes [bin][k][row] (conjugation folded into the sign of the
+// imaginary plane) while the next slice is already in flight in registers; each
+// wave then issues v_mfma_f32_32x32x2_f32, four real products per complex
+// product: Cre += Ar*Br + (-Ai)*Bi, Cim += Ar*Bi + Ai*Br.  C leaves through LDS
+// so that stores cover whole runs.  Only this contraction uses MFMA; it is the
+// one dense product of the convolution path.
 #include "common.h"
 
 namespace fbfft_amd {
@@ -24,11 +27,13 @@ namespace {
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
-constexpr int TI = 32, TJ = 32, XB = 16, KC = 4, THREADS = 256;  // 4 waves
-constexpr int XS = KC * 32 + 4;              // bin stride of an LDS plane (dwords), padded
-constexpr int PLANE = XB * XS;               // one of Ar, Ai, Br, Bi
-constexpr int CSTR = XB + 1;                 // padded bin stride of the C staging buffer (complex)
-constexpr int LDS_FLOATS = (4 * PLANE > 8 * 32 * CSTR * 2) ? 4 * PLANE : 8 * 32 * CSTR * 2;
+constexpr int TI = 64, TJ = 64, XB = 8, KC = 4, THREADS = 512;  // 8 waves, one bin each
+constexpr int XS = KC * 64 + 4;   // bin stride of an LDS plane (dwords): the 4 bin pairs a
+                                  // half-wave writes land 8 banks apart
+constexpr int PLANE = XB * XS;    // one of Ar, Ai, Br, Bi
+constexpr int CSTR = XB + 1;      // padded bin stride of the C staging buffer (complex)
+constexpr int STAGE_FLOATS = 8 * TJ * CSTR * 2;
+constexpr int LDS_FLOATS = (4 * PLANE > STAGE_FLOATS) ? 4 * PLANE : STAGE_FLOATS;
 
 struct MMArgs {
   const float* A;
@@ -45,11 +50,11 @@ struct MMArgs {
   int chunks;  // ceil(XY / XB)
 };
 
-// 16 bins x 4 k x 32 rows of one operand: each lane fetches two float4 (bins
-// 2p, 2p+1 of two (row, k) elements).  Lanes of a wave: p = lane % 8 walks the
-// line, lane / 8 walks 8 consecutive rows.
+// One slice of one operand: 64 rows x KC k x 8 bins.  Lane t fetches bins 2p, 2p+1
+// (p = t % 4) of row (t/4) % 64 at k = (t/4)/64 + 2u: within a wave
+// 16 consecutive rows, 64 bytes each.
 struct Fetch {
-  float4 v[2];
+  float4 v[KC / 2];
 };
 
 template <bool VEC4>
@@ -57,18 +62,14 @@ __device__ __forceinline__ Fetch fetchSlice(const float* base, long rowStride, l
                                             int rows, int row0, int K, int k0, int XY, int x0,
                                             int t) {
   Fetch f;
-  const int p = t % 8;
+  const int p = t % 4;
   const int x = x0 + 2 * p;
-  f.v[0] = float4{0.f, 0.f, 0.f, 0.f};
-  f.v[1] = float4{0.f, 0.f, 0.f, 0.f};
-  // element e = lane/8 + 32u -> row = e % 32, kk = e / 32: one call covers two
-  // values of k; the caller issues a second call for k0 + 2
+  const int e = t / 4;
+  const int row = row0 + e % 64;
 #pragma unroll
-  for (int u = 0; u < 2; ++u) {
-    const int e = t / 8 + 32 * u;
-    const int r = e % 32;
-    const int kk = e / 32;  // 0 or 1 (+2 by the caller through k0)
-    const int row = row0 + r, k = k0 + kk;
+  for (int u = 0; u < KC / 2; ++u) {
+    const int k = k0 + e / 64 + 2 * u;
+    f.v[u] = float4{0.f, 0.f, 0.f, 0.f};
     if (row < rows && k < K && x < XY) {
       const float* src = base + (long)row * rowStride + (long)k * kStride + 2L * x;
       if (VEC4 && x + 1 < XY) {
@@ -88,14 +89,12 @@ __device__ __forceinline__ Fetch fetchSlice(const float* base, long rowStride, l
   return f;
 }
 
-__device__ __forceinline__ void stashSlice(float* re, float* im, const Fetch& f, float sign, int kBase,
-                                           int t) {
-  const int p = t % 8;
+__device__ __forceinline__ void stashSlice(float* re, float* im, const Fetch& f, float sign, int t) {
+  const int p = t % 4;
+  const int e = t / 4;
 #pragma unroll
-  for (int u = 0; u < 2; ++u) {
-    const int e = t / 8 + 32 * u;
-    const int r = e % 32, kk = kBase + e / 32;
-    const int o = kk * 32 + r;
+  for (int u = 0; u < KC / 2; ++u) {
+    const int o = (e / 64 + 2 * u) * 64 + e % 64;
     re[(2 * p) * XS + o] = f.v[u].x;
     im[(2 * p) * XS + o] = sign * f.v[u].y;
     re[(2 * p + 1) * XS + o] = f.v[u].z;
@@ -104,7 +103,7 @@ __device__ __forceinline__ void stashSlice(float* re, float* im, const Fetch& f,
 }
 
 template <bool VEC4>
-__global__ __launch_bounds__(THREADS, 2) void transposeMMKernel(MMArgs a) {
+__global__ __launch_bounds__(THREADS) void transposeMMKernel(MMArgs a) {
   __shared__ __align__(8) float lds[LDS_FLOATS];
   float* Ar = lds;
   float* Ai = lds + PLANE;
@@ -115,7 +114,8 @@ __global__ __launch_bounds__(THREADS, 2) void transposeMMKernel(MMArgs a) {
   const int lane = t % 64, w = t / 64;
   // Workgroups are dealt round-robin to the 8 XCDs, each with its own L2.  Give
   // every XCD a contiguous range of logical ids, ordered bin-chunk first, so that
-  // all (i, j) tiles that re-read the same lines of A and B share one L2.
+  // the tiles that re-read the same lines of A and B (and the two chunks that
+  // share a 128-byte line) meet in one L2.
   const int tilesJ = (a.J + TJ - 1) / TJ, tilesI = (a.I + TI - 1) / TI;
   const int total = a.chunks * tilesI * tilesJ;
   const int per = (total + 7) / 8;
@@ -126,85 +126,97 @@ __global__ __launch_bounds__(THREADS, 2) void transposeMMKernel(MMArgs a) {
   const int j0 = (rem % tilesJ) * TJ;
   const int i0 = (rem / tilesJ) * TI;
 
-  floatx16 cre[4], cim[4];
+  // sub-tile (si, sj): rows 32*si.., columns 32*sj..
+  floatx16 cre[2][2], cim[2][2];
 #pragma unroll
-  for (int b = 0; b < 4; ++b)
+  for (int si = 0; si < 2; ++si)
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      cre[b][r] = 0.f;
-      cim[b][r] = 0.f;
-    }
+    for (int sj = 0; sj < 2; ++sj)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        cre[si][sj][r] = 0.f;
+        cim[si][sj][r] = 0.f;
+      }
 
-  // slice = KC = 4 values of k: two fetches (k0, k0+1) and (k0+2, k0+3) per operand
-  Fetch fa0, fa1, fb0, fb1;
+  Fetch fa, fb;
   auto fetchAll = [&](int k0) {
-    fa0 = fetchSlice<VEC4>(a.A, a.aRow, a.aK, a.I, i0, a.K, k0, a.XY, x0, t);
-    fa1 = fetchSlice<VEC4>(a.A, a.aRow, a.aK, a.I, i0, a.K, k0 + 2, a.XY, x0, t);
-    fb0 = fetchSlice<VEC4>(a.B, a.bCol, a.bK, a.J, j0, a.K, k0, a.XY, x0, t);
-    fb1 = fetchSlice<VEC4>(a.B, a.bCol, a.bK, a.J, j0, a.K, k0 + 2, a.XY, x0, t);
+    fa = fetchSlice<VEC4>(a.A, a.aRow, a.aK, a.I, i0, a.K, k0, a.XY, x0, t);
+    fb = fetchSlice<VEC4>(a.B, a.bCol, a.bK, a.J, j0, a.K, k0, a.XY, x0, t);
   };
   fetchAll(0);
+  const int xo = w * XS + lane % 32 + 64 * (lane / 32);  // bin w, row/col lane%32, k parity lane/32
   for (int k0 = 0; k0 < a.K; k0 += KC) {
     __syncthreads();  // previous slice fully consumed
-    stashSlice(Ar, Ai, fa0, a.aSign, 0, t);
-    stashSlice(Ar, Ai, fa1, a.aSign, 2, t);
-    stashSlice(Br, Bi, fb0, a.bSign, 0, t);
-    stashSlice(Br, Bi, fb1, a.bSign, 2, t);
+    stashSlice(Ar, Ai, fa, a.aSign, t);
+    stashSlice(Br, Bi, fb, a.bSign, t);
     __syncthreads();
     if (k0 + KC < a.K) fetchAll(k0 + KC);
 #pragma unroll
-    for (int b = 0; b < 4; ++b) {
-      const int xo = (4 * w + b) * XS;
+    for (int s = 0; s < KC / 2; ++s) {
+      // the lane supplies row/col lane%32 (+32 for the second sub-tile) at k = 2s + lane/32
+      const int o = xo + s * 128;
+      float ar[2], ai[2], br[2], bi[2];
 #pragma unroll
-      for (int s = 0; s < KC / 2; ++s) {
-        // lane supplies row/col lane%32 at k = 2s + lane/32: 64 consecutive dwords
-        const int o = xo + s * 64 + lane;
-        const float ar = Ar[o], ai = Ai[o], br = Br[o], bi = Bi[o];
-        cre[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(ar, br, cre[b], 0, 0, 0);
-        cre[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(-ai, bi, cre[b], 0, 0, 0);
-        cim[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(ar, bi, cim[b], 0, 0, 0);
-        cim[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(ai, br, cim[b], 0, 0, 0);
+      for (int q = 0; q < 2; ++q) {
+        ar[q] = Ar[o + 32 * q];
+        ai[q] = Ai[o + 32 * q];
+        br[q] = Br[o + 32 * q];
+        bi[q] = Bi[o + 32 * q];
       }
+#pragma unroll
+      for (int si = 0; si < 2; ++si)
+#pragma unroll
+        for (int sj = 0; sj < 2; ++sj) {
+          cre[si][sj] = __builtin_amdgcn_mfma_f32_32x32x2f32(ar[si], br[sj], cre[si][sj], 0, 0, 0);
+          cim[si][sj] = __builtin_amdgcn_mfma_f32_32x32x2f32(ar[si], bi[sj], cim[si][sj], 0, 0, 0);
+        }
+#pragma unroll
+      for (int si = 0; si < 2; ++si)
+#pragma unroll
+        for (int sj = 0; sj < 2; ++sj) {
+          cre[si][sj] = __builtin_amdgcn_mfma_f32_32x32x2f32(-ai[si], bi[sj], cre[si][sj], 0, 0, 0);
+          cim[si][sj] = __builtin_amdgcn_mfma_f32_32x32x2f32(ai[si], br[sj], cim[si][sj], 0, 0, 0);
+        }
     }
   }
 
-  // ---- epilogue: C leaves through LDS so that every store covers whole 128-byte
-  // runs (the 16 bins of one (i, j) element); written straight from the
-  // accumulators each lane would scatter 8-byte pieces 4 KB apart.
-  // Register r of lane l holds row 8*(r/4) + 4*(l/32) + r%4, column l%32, so the
-  // four registers 4c..4c+3 of all lanes form rows 8c..8c+7: one chunk.
-  float2* stage = reinterpret_cast<float2*>(lds);  // [8 rows][32 cols][CSTR] complex
+  // ---- epilogue: C leaves through LDS so that every store covers whole runs (the
+  // 8 bins of one (i, j) element).  Register r of lane l holds row
+  // 8*(r/4) + 4*(l/32) + r%4 and column l%32 of a sub-tile, so registers 4c..4c+3 of
+  // all lanes form rows 8c..8c+7 of a sub-tile row: one chunk of 8 rows x 64 columns.
+  float2* stage = reinterpret_cast<float2*>(lds);  // [8 rows][64 cols][CSTR] complex
   const int col = lane % 32, hh = lane / 32;
 #pragma unroll
-  for (int c = 0; c < 4; ++c) {
-    __syncthreads();  // operand slices / previous chunk fully consumed
+  for (int si = 0; si < 2; ++si)
 #pragma unroll
-    for (int rr = 0; rr < 4; ++rr) {
-      const int row = 4 * hh + rr;
+    for (int c = 0; c < 4; ++c) {
+      __syncthreads();  // operand slices / previous chunk fully consumed
 #pragma unroll
-      for (int b = 0; b < 4; ++b)
-        stage[(row * 32 + col) * CSTR + 4 * w + b] = float2{cre[b][4 * c + rr], cim[b][4 * c + rr]};
-    }
-    __syncthreads();
-    // 256 (row, col) elements x 16 bins: 16 lanes per element, 16 elements per pass
-    const int xl = t % 16;
+      for (int sj = 0; sj < 2; ++sj)
 #pragma unroll
-    for (int pass = 0; pass < 16; ++pass) {
-      const int e = t / 16 + 16 * pass;  // 0..255
-      const int row = e / 32, cc = e % 32;
-      const int i = i0 + 8 * c + row, j = j0 + cc, x = x0 + xl;
-      if (i < a.I && j < a.J && x < a.XY) {
-        float2 acc = stage[(row * 32 + cc) * CSTR + xl];
-        float* dst = a.C + (long)i * a.cRow + (long)j * a.cCol + 2L * x;
-        if (a.accumulate) {
-          float2 old = *reinterpret_cast<const float2*>(dst);
-          acc.x += old.x;
-          acc.y += old.y;
+        for (int rr = 0; rr < 4; ++rr)
+          stage[((4 * hh + rr) * TJ + 32 * sj + col) * CSTR + w] =
+              float2{cre[si][sj][4 * c + rr], cim[si][sj][4 * c + rr]};
+      __syncthreads();
+      // 512 (row, col) elements x 8 bins: 8 lanes per element, 64 elements per pass
+      const int xl = t % 8;
+#pragma unroll
+      for (int pass = 0; pass < 8; ++pass) {
+        const int e = t / 8 + 64 * pass;  // 0..511
+        const int row = e / TJ, cc = e % TJ;
+        const int i = i0 + 32 * si + 8 * c + row, j = j0 + cc, x = x0 + xl;
+        if (i < a.I && j < a.J && x < a.XY) {
+          float2 acc = stage[(row * TJ + cc) * CSTR + xl];
+          float* dst = a.C + (long)i * a.cRow + (long)j * a.cCol + 2L * x;
+          if (a.accumulate) {
+            float2 old = *reinterpret_cast<const float2*>(dst);
+            acc.x += old.x;
+            acc.y += old.y;
+          }
+          *reinterpret_cast<float2*>(dst) = float2{acc.x * a.invNorm, acc.y * a.invNorm};
         }
-        *reinterpret_cast<float2*>(dst) = float2{acc.x * a.invNorm, acc.y * a.invNorm};
       }
     }
-  }
 }
 
 }  // namespace
