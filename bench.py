@@ -163,7 +163,7 @@ def run_only(name, steps, warmup, F, synth, torch, dev):
     """One workload in a tight loop, for profiling."""
     if name in ("r2c32", "c2r32", "r2c64", "c2r64", "r2c128", "c2r128"):
         n = int(name[3:])
-        b = {32: 16384, 64: 16384, 128: 4096}[n]
+        b = int(os.environ.get("FBFFT_BENCH_B", {32: 16384, 64: 16384, 128: 4096}[n]))
         x = synth.normal((b, n, n), seed=1, device=dev)
         spec = torch.empty((b, n // 2 + 1, n, 2), device=dev)
         fwd = prepared("fbfft_r2c_2d", F, x, spec, 0, 0)

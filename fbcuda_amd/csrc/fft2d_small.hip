@@ -41,7 +41,11 @@ struct SmallCfg {
 // FAST_REAL: real is [B][N][N] with unit x stride, even row/batch strides,
 //            8-byte aligned base and zero padding -> 8-byte vector accesses.
 // FAST_CPLX: each spectrum plane is contiguous and 16-byte aligned.
-template <int N, bool FAST_REAL, bool FAST_CPLX>
+// GPW:       groups of P planes a wave processes (1 or 2).  With 2, the loads of
+//            the second group are issued as soon as the first group's columns
+//            have left the registers, so they fly under the first group's row
+//            pass and stores: the wave pays the HBM latency once instead of twice.
+template <int N, bool FAST_REAL, bool FAST_CPLX, int GPW>
 __global__ __launch_bounds__(64) void fft2dSmallForward(RealView real, CplxView cplx, int padL,
                                                         int padU) {
   using C = SmallCfg<N>;
@@ -51,71 +55,85 @@ __global__ __launch_bounds__(64) void fft2dSmallForward(RealView real, CplxView 
   const int lane = threadIdx.x;
   const int pl = lane / T;
   const int l = lane % T;
-  const int b0 = blockIdx.x * P;
   const int B = real.B;
-  const int b = min(b0 + pl, B - 1);  // tail lanes redo the last plane and skip the store
-
-  // ---- column pass ----
-  c32 z0[H], z1[H];
-  if constexpr (FAST_REAL) {
-    const float2* src = reinterpret_cast<const float2*>(real.data + (size_t)b * real.sb) + l;
-    const int rs2 = real.sy / 2;
-    staticFor<H>([&](auto jj) {
-      constexpr int j = decltype(jj)::value;
-      float2 r0 = src[(size_t)(2 * j) * rs2];
-      float2 r1 = src[(size_t)(2 * j + 1) * rs2];
-      z0[j] = c32{r0.x, r1.x};
-      z1[j] = c32{r0.y, r1.y};
-    });
-  } else {
-    loadColumnsWindow<N>(real.data + (size_t)b * real.sb, real.sy, real.sx, real.h, real.w, padL,
-                         padU, l, z0, z1);
-  }
   c32* plane = lds + pl * PS;
-  columnPassForward<N>(z0, z1, plane, l);
-  __syncthreads();
 
-  // ---- row pass: lane l owns packed row l ----
+  auto load = [&](int b0, c32 (&z0)[H], c32 (&z1)[H]) __attribute__((always_inline)) {
+    const int b = min(b0 + pl, B - 1);  // tail lanes redo the last plane and skip the store
+    if constexpr (FAST_REAL) {
+      const float2* src = reinterpret_cast<const float2*>(real.data + (size_t)b * real.sb) + l;
+      const int rs2 = real.sy / 2;
+      staticFor<H>([&](auto jj) {
+        constexpr int j = decltype(jj)::value;
+        float2 r0 = src[(size_t)(2 * j) * rs2];
+        float2 r1 = src[(size_t)(2 * j + 1) * rs2];
+        z0[j] = c32{r0.x, r1.x};
+        z1[j] = c32{r0.y, r1.y};
+      });
+    } else {
+      loadColumnsWindow<N>(real.data + (size_t)b * real.sb, real.sy, real.sx, real.h, real.w, padL,
+                           padU, l, z0, z1);
+    }
+  };
+
+  // copy out: (H+1) x N complex per plane, rows 0 and H unpacked from packed row 0
+  auto copyOut = [&](int b0) __attribute__((always_inline)) {
+    staticFor<C::ITERS>([&](auto tt) {
+      constexpr int t = decltype(tt)::value;
+      const int q = lane + 64 * t;
+      const int pp = q / C::F4_PER_PLANE;
+      const int rem = q % C::F4_PER_PLANE;
+      const int r = rem / (N / 2);
+      const int kx = 2 * (rem % (N / 2));
+      const c32* base = lds + pp * PS;
+      float4 v;
+      if (r == 0 || r == H) {
+        c32 a0 = base[kx], a1 = base[kx + 1];
+        c32 m0 = base[(N - kx) & (N - 1)], m1 = base[N - kx - 1];
+        if (r == 0) {
+          v = float4{0.5f * (a0.x + m0.x), 0.5f * (a0.y - m0.y), 0.5f * (a1.x + m1.x),
+                     0.5f * (a1.y - m1.y)};
+        } else {
+          v = float4{0.5f * (a0.y + m0.y), 0.5f * (m0.x - a0.x), 0.5f * (a1.y + m1.y),
+                     0.5f * (m1.x - a1.x)};
+        }
+      } else {
+        v = ldsLoad4(base + r * RS + kx);
+      }
+      const int bo = b0 + pp;
+      if (bo < B) {
+        if constexpr (FAST_CPLX) {
+          reinterpret_cast<float4*>(cplx.data + (size_t)bo * cplx.sb)[rem] = v;
+        } else {
+          float* o = cplx.data + (size_t)bo * cplx.sb + (size_t)r * cplx.sr + (size_t)kx * cplx.sc;
+          *reinterpret_cast<float2*>(o) = float2{v.x, v.y};
+          *reinterpret_cast<float2*>(o + cplx.sc) = float2{v.z, v.w};
+        }
+      }
+    });
+  };
+
+  const int g0 = blockIdx.x * GPW * P;
+  c32 za0[H], za1[H];
+  load(g0, za0, za1);
+  columnPassForward<N>(za0, za1, plane, l);
+  __syncthreads();
+  c32 zb0[H], zb1[H];
+  if constexpr (GPW == 2) load(g0 + P, zb0, zb1);
   rowPassInPlace<N, true>(plane, l);
   __syncthreads();
-
-  // ---- copy out: (H+1) x N complex per plane, rows 0 and H unpacked from packed row 0 ----
-  staticFor<C::ITERS>([&](auto tt) {
-    constexpr int t = decltype(tt)::value;
-    const int q = lane + 64 * t;
-    const int pp = q / C::F4_PER_PLANE;
-    const int rem = q % C::F4_PER_PLANE;
-    const int r = rem / (N / 2);
-    const int kx = 2 * (rem % (N / 2));
-    const c32* base = lds + pp * PS;
-    float4 v;
-    if (r == 0 || r == H) {
-      c32 a0 = base[kx], a1 = base[kx + 1];
-      c32 m0 = base[(N - kx) & (N - 1)], m1 = base[N - kx - 1];
-      if (r == 0) {
-        v = float4{0.5f * (a0.x + m0.x), 0.5f * (a0.y - m0.y), 0.5f * (a1.x + m1.x),
-                   0.5f * (a1.y - m1.y)};
-      } else {
-        v = float4{0.5f * (a0.y + m0.y), 0.5f * (m0.x - a0.x), 0.5f * (a1.y + m1.y),
-                   0.5f * (m1.x - a1.x)};
-      }
-    } else {
-      v = ldsLoad4(base + r * RS + kx);
-    }
-    const int bo = b0 + pp;
-    if (bo < B) {
-      if constexpr (FAST_CPLX) {
-        reinterpret_cast<float4*>(cplx.data + (size_t)bo * cplx.sb)[rem] = v;
-      } else {
-        float* o = cplx.data + (size_t)bo * cplx.sb + (size_t)r * cplx.sr + (size_t)kx * cplx.sc;
-        *reinterpret_cast<float2*>(o) = float2{v.x, v.y};
-        *reinterpret_cast<float2*>(o + cplx.sc) = float2{v.z, v.w};
-      }
-    }
-  });
+  copyOut(g0);
+  if constexpr (GPW == 2) {
+    __syncthreads();
+    columnPassForward<N>(zb0, zb1, plane, l);
+    __syncthreads();
+    rowPassInPlace<N, true>(plane, l);
+    __syncthreads();
+    copyOut(g0 + P);
+  }
 }
 
-template <int N, bool FAST_REAL, bool FAST_CPLX>
+template <int N, bool FAST_REAL, bool FAST_CPLX, int GPW>
 __global__ __launch_bounds__(64) void fft2dSmallInverse(CplxView cplx, RealView real, int padL,
                                                         int padU) {
   using C = SmallCfg<N>;
@@ -125,71 +143,123 @@ __global__ __launch_bounds__(64) void fft2dSmallInverse(CplxView cplx, RealView 
   const int lane = threadIdx.x;
   const int pl = lane / T;
   const int l = lane % T;
-  const int b0 = blockIdx.x * P;
   const int B = real.B;
-
-  // ---- copy in: natural [row][kx] order ----
-  staticFor<C::ITERS>([&](auto tt) {
-    constexpr int t = decltype(tt)::value;
-    const int q = lane + 64 * t;
-    const int pp = q / C::F4_PER_PLANE;
-    const int rem = q % C::F4_PER_PLANE;
-    const int r = rem / (N / 2);
-    const int kx = 2 * (rem % (N / 2));
-    const int bi = min(b0 + pp, B - 1);
-    float4 v;
-    if constexpr (FAST_CPLX) {
-      v = reinterpret_cast<const float4*>(cplx.data + (size_t)bi * cplx.sb)[rem];
-    } else {
-      const float* o = cplx.data + (size_t)bi * cplx.sb + (size_t)r * cplx.sr + (size_t)kx * cplx.sc;
-      float2 a = *reinterpret_cast<const float2*>(o);
-      float2 c = *reinterpret_cast<const float2*>(o + cplx.sc);
-      v = float4{a.x, a.y, c.x, c.y};
-    }
-    *reinterpret_cast<float4*>(lds + pp * PS + r * RS + kx) = v;
-  });
-  __syncthreads();
-
-  // ---- pack rows 0 and H into one complex row: Q = F0 + i*FH.  At kx = 0 only
-  // the real parts are used, as in the reference (fbfft/FFT2D32.cuh:310-316). ----
-  {
-    c32* r0 = lds + pl * PS + 2 * l;
-    const c32* rH = r0 + H * RS;
-    float4 a = ldsLoad4(r0);
-    float4 c = ldsLoad4(rH);
-    float4 q = float4{a.x - c.y, a.y + c.x, a.z - c.w, a.w + c.z};
-    if (l == 0) {
-      q.x = a.x;
-      q.y = c.x;
-    }
-    *reinterpret_cast<float4*>(r0) = q;
-  }
-  __syncthreads();
-
-  // ---- row pass (inverse) ----
   c32* plane = lds + pl * PS;
-  rowPassInPlace<N, false>(plane, l);
-  __syncthreads();
 
-  // ---- column pass (inverse): lane l owns columns 2l, 2l+1 ----
-  c32 z0[H], z1[H];
-  columnPassInverse<N>(plane, l, z0, z1);
-
-  const int b = b0 + pl;
-  if (b >= B) return;
-  if constexpr (FAST_REAL) {
-    float2* dst = reinterpret_cast<float2*>(real.data + (size_t)b * real.sb) + l;
-    const int rs2 = real.sy / 2;
-    staticFor<H>([&](auto jj) {
-      constexpr int j = decltype(jj)::value;
-      c32 a = z0[slot<H>(j)], c = z1[slot<H>(j)];
-      dst[(size_t)(2 * j) * rs2] = float2{a.x, c.x};
-      dst[(size_t)(2 * j + 1) * rs2] = float2{a.y, c.y};
+  // spectra of one group, natural [row][kx] order, one float4 per lane per step
+  float in[GPW][4 * C::ITERS];  // plain floats: always promoted to registers
+  auto load = [&](auto gg, int b0) __attribute__((always_inline)) {
+    constexpr int G = decltype(gg)::value;
+    staticFor<C::ITERS>([&](auto tt) {
+      constexpr int t = decltype(tt)::value;
+      const int q = lane + 64 * t;
+      const int pp = q / C::F4_PER_PLANE;
+      const int rem = q % C::F4_PER_PLANE;
+      const int bi = min(b0 + pp, B - 1);
+      if constexpr (FAST_CPLX) {
+        const float4 v = reinterpret_cast<const float4*>(cplx.data + (size_t)bi * cplx.sb)[rem];
+        in[G][4 * t] = v.x;
+        in[G][4 * t + 1] = v.y;
+        in[G][4 * t + 2] = v.z;
+        in[G][4 * t + 3] = v.w;
+      } else {
+        const int r = rem / (N / 2), kx = 2 * (rem % (N / 2));
+        const float* o = cplx.data + (size_t)bi * cplx.sb + (size_t)r * cplx.sr + (size_t)kx * cplx.sc;
+        float2 a = *reinterpret_cast<const float2*>(o);
+        float2 c = *reinterpret_cast<const float2*>(o + cplx.sc);
+        in[G][4 * t] = a.x;
+        in[G][4 * t + 1] = a.y;
+        in[G][4 * t + 2] = c.x;
+        in[G][4 * t + 3] = c.y;
+      }
     });
+  };
+
+  auto process = [&](auto gg, int b0) __attribute__((always_inline)) {
+    constexpr int G = decltype(gg)::value;
+    staticFor<C::ITERS>([&](auto tt) {
+      constexpr int t = decltype(tt)::value;
+      const int q = lane + 64 * t;
+      const int pp = q / C::F4_PER_PLANE;
+      const int rem = q % C::F4_PER_PLANE;
+      *reinterpret_cast<float4*>(lds + pp * PS + (rem / (N / 2)) * RS + 2 * (rem % (N / 2))) =
+          float4{in[G][4 * t], in[G][4 * t + 1], in[G][4 * t + 2], in[G][4 * t + 3]};
+    });
+    __syncthreads();
+    // pack rows 0 and H into one complex row: Q = F0 + i*FH.  At kx = 0 only the real
+    // parts are used, as in the reference (fbfft/FFT2D32.cuh:310-316).
+    {
+      c32* r0 = plane + 2 * l;
+      const c32* rH = r0 + H * RS;
+      float4 a = ldsLoad4(r0);
+      float4 c = ldsLoad4(rH);
+      float4 q = float4{a.x - c.y, a.y + c.x, a.z - c.w, a.w + c.z};
+      if (l == 0) {
+        q.x = a.x;
+        q.y = c.x;
+      }
+      *reinterpret_cast<float4*>(r0) = q;
+    }
+    __syncthreads();
+    rowPassInPlace<N, false>(plane, l);
+    __syncthreads();
+    c32 z0[H], z1[H];
+    columnPassInverse<N>(plane, l, z0, z1);
+    const int b = b0 + pl;
+    if (b < B) {
+      if constexpr (FAST_REAL) {
+        float2* dst = reinterpret_cast<float2*>(real.data + (size_t)b * real.sb) + l;
+        const int rs2 = real.sy / 2;
+        staticFor<H>([&](auto jj) {
+          constexpr int j = decltype(jj)::value;
+          c32 a = z0[slot<H>(j)], c = z1[slot<H>(j)];
+          dst[(size_t)(2 * j) * rs2] = float2{a.x, c.x};
+          dst[(size_t)(2 * j + 1) * rs2] = float2{a.y, c.y};
+        });
+      } else {
+        storeColumnsWindow<N>(real.data + (size_t)b * real.sb, real.sy, real.sx, real.h, real.w,
+                              padL, padU, l, z0, z1, 1.0f);
+      }
+    }
+  };
+
+  const int g0 = blockIdx.x * GPW * P;
+  constexpr std::integral_constant<int, 0> first{};
+  load(first, g0);
+  if constexpr (GPW == 2) {
+    constexpr std::integral_constant<int, 1> second{};
+    load(second, g0 + P);  // in flight while the first group is transformed
+    process(first, g0);
+    __syncthreads();
+    process(second, g0 + P);
   } else {
-    storeColumnsWindow<N>(real.data + (size_t)b * real.sb, real.sy, real.sx, real.h, real.w, padL,
-                          padU, l, z0, z1, 1.0f);
+    process(first, g0);
   }
+}
+
+// Two groups per wave pay off only when the launch would otherwise take between
+// one and two rounds of resident waves: then the second round's load latency is
+// exposed, and folding it into the first round's waves (with their loads already
+// in flight) hides it.  Measured on 32 x 32 R2C: 26.9 -> 24.6 us at 16384 planes,
+// but 102 -> 113 us at 65536 planes, where other waves already cover the latency.
+int computeUnits() {
+  static const int n = [] {
+    int dev = 0, cus = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
+        cus <= 0)
+      cus = 256;
+    return cus;
+  }();
+  return n;
+}
+
+template <int N>
+bool pairGroups(int groups) {
+  constexpr int ldsBytes = SmallCfg<N>::P * SmallCfg<N>::PS * (int)sizeof(c32);
+  constexpr int wavesPerCU = (160 * 1024 / ldsBytes) < 32 ? (160 * 1024 / ldsBytes) : 32;
+  const int slots = computeUnits() * wavesPerCU;
+  return groups > slots && groups <= 2 * slots;
 }
 
 bool fastReal(int N, const RealView& r, int padL, int padU) {
@@ -204,32 +274,60 @@ bool fastCplx(int N, const CplxView& c) {
 template <int N>
 int launchForward(const RealView& real, const CplxView& cplx, int padL, int padU, hipStream_t s) {
   using C = SmallCfg<N>;
-  dim3 grid(ceilDiv(real.B, C::P)), block(64);
+  const int groups = ceilDiv(real.B, C::P);
   const bool fr = fastReal(N, real, padL, padU), fc = fastCplx(N, cplx);
-  if (fr && fc)
-    fft2dSmallForward<N, true, true><<<grid, block, 0, s>>>(real, cplx, padL, padU);
-  else if (fc)
-    fft2dSmallForward<N, false, true><<<grid, block, 0, s>>>(real, cplx, padL, padU);
-  else if (fr)
-    fft2dSmallForward<N, true, false><<<grid, block, 0, s>>>(real, cplx, padL, padU);
-  else
-    fft2dSmallForward<N, false, false><<<grid, block, 0, s>>>(real, cplx, padL, padU);
+  dim3 block(64);
+  if (pairGroups<N>(groups)) {
+    dim3 grid(ceilDiv(groups, 2));
+    if (fr && fc)
+      fft2dSmallForward<N, true, true, 2><<<grid, block, 0, s>>>(real, cplx, padL, padU);
+    else if (fc)
+      fft2dSmallForward<N, false, true, 2><<<grid, block, 0, s>>>(real, cplx, padL, padU);
+    else if (fr)
+      fft2dSmallForward<N, true, false, 2><<<grid, block, 0, s>>>(real, cplx, padL, padU);
+    else
+      fft2dSmallForward<N, false, false, 2><<<grid, block, 0, s>>>(real, cplx, padL, padU);
+  } else {
+    dim3 grid(groups);
+    if (fr && fc)
+      fft2dSmallForward<N, true, true, 1><<<grid, block, 0, s>>>(real, cplx, padL, padU);
+    else if (fc)
+      fft2dSmallForward<N, false, true, 1><<<grid, block, 0, s>>>(real, cplx, padL, padU);
+    else if (fr)
+      fft2dSmallForward<N, true, false, 1><<<grid, block, 0, s>>>(real, cplx, padL, padU);
+    else
+      fft2dSmallForward<N, false, false, 1><<<grid, block, 0, s>>>(real, cplx, padL, padU);
+  }
   return launchStatus();
 }
 
 template <int N>
 int launchInverse(const CplxView& cplx, const RealView& real, int padL, int padU, hipStream_t s) {
   using C = SmallCfg<N>;
-  dim3 grid(ceilDiv(real.B, C::P)), block(64);
+  const int groups = ceilDiv(real.B, C::P);
   const bool fr = fastReal(N, real, padL, padU), fc = fastCplx(N, cplx);
-  if (fr && fc)
-    fft2dSmallInverse<N, true, true><<<grid, block, 0, s>>>(cplx, real, padL, padU);
-  else if (fc)
-    fft2dSmallInverse<N, false, true><<<grid, block, 0, s>>>(cplx, real, padL, padU);
-  else if (fr)
-    fft2dSmallInverse<N, true, false><<<grid, block, 0, s>>>(cplx, real, padL, padU);
-  else
-    fft2dSmallInverse<N, false, false><<<grid, block, 0, s>>>(cplx, real, padL, padU);
+  dim3 block(64);
+  if (pairGroups<N>(groups)) {
+    dim3 grid(ceilDiv(groups, 2));
+    if (fr && fc)
+      fft2dSmallInverse<N, true, true, 2><<<grid, block, 0, s>>>(cplx, real, padL, padU);
+    else if (fc)
+      fft2dSmallInverse<N, false, true, 2><<<grid, block, 0, s>>>(cplx, real, padL, padU);
+    else if (fr)
+      fft2dSmallInverse<N, true, false, 2><<<grid, block, 0, s>>>(cplx, real, padL, padU);
+    else
+      fft2dSmallInverse<N, false, false, 2><<<grid, block, 0, s>>>(cplx, real, padL, padU);
+  } else {
+    dim3 grid(groups);
+    if (fr && fc)
+      fft2dSmallInverse<N, true, true, 1><<<grid, block, 0, s>>>(cplx, real, padL, padU);
+    else if (fc)
+      fft2dSmallInverse<N, false, true, 1><<<grid, block, 0, s>>>(cplx, real, padL, padU);
+    else if (fr)
+      fft2dSmallInverse<N, true, false, 1><<<grid, block, 0, s>>>(cplx, real, padL, padU);
+    else
+      fft2dSmallInverse<N, false, false, 1><<<grid, block, 0, s>>>(cplx, real, padL, padU);
+  }
   return launchStatus();
 }
 

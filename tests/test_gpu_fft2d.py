@@ -133,3 +133,22 @@ def test_full_size_properties(oracle, N, B):
     torch.cuda.synchronize()
     lin = (sz - (2 * spec[:n] + spec[n:2 * n])).double().norm() / sz.double().norm()
     assert float(lin) < TOL_FFT
+
+
+@pytest.mark.parametrize("N,B", [(32, 9001), (16, 33333), (8, 110001)])
+def test_two_groups_per_wave_tail(oracle, N, B):
+    """Batch sizes in the one-to-two-round regime, where a wave transforms two groups
+    of planes and prefetches the second: odd group counts and a ragged last group."""
+    d = dev()
+    x = synth.normal((B, N, N), seed=12, device=d)
+    spec = torch.full((B, N // 2 + 1, N, 2), float("nan"), device=d)
+    back = torch.full((B, N, N), float("nan"), device=d)
+    assert F.fbfft2D(x, spec) == F.Success
+    assert F.fbifft2D(spec, back) == F.Success
+    torch.cuda.synchronize()
+    assert bool(torch.isfinite(spec).all()) and bool(torch.isfinite(back).all())
+    err = (back / (N * N) - x).double().norm() / x.double().norm()
+    assert float(err) < TOL_FFT
+    pick = [0, 1, B // 2, B - 130, B - 5, B - 4, B - 3, B - 2, B - 1]
+    _, want = oracle.fbfft2d(x[pick].cpu().numpy(), N)
+    assert rel(spec[pick].cpu().numpy(), want) < TOL_FFT
