@@ -10,18 +10,16 @@
 //   1. forwardBinMajor:  planes -> S[bin][k][row]   (row = image / output plane)
 //      a 256-lane workgroup transforms SLOTS = 512/N planes with consecutive
 //      `row` and the same k and writes each bin as one contiguous run.
-//   2. binGemm:          C[bin][i][j] = invNorm * sum_k A[bin][k][i] * conj(B[bin][k][j])
+//   2. binGemmDirect:    C[bin][i][j] = invNorm * sum_k A[bin][k][i] * conj(B[bin][k][j])
 //      one workgroup = one bin x (128 x 64) tile; k-slices of A and B are
-//      contiguous in HBM and are copied verbatim into LDS; 4 waves x 2 MFMA
-//      32x32x2 sub-tiles x (re, im); every spectrum element is fetched from HBM
-//      once per j-tile and C is written once with coalesced stores.  Workgroup
-//      ids are remapped so that the j-tiles of a bin run on the same XCD (shared L2).
+//      contiguous in HBM and are copied verbatim into LDS by global_load_lds;
+//      4 waves x 2 MFMA 32x32x2 sub-tiles x (re, im); counters show A + B fetched
+//      from HBM exactly once (the three j-tiles of a bin share an L2: workgroup ids
+//      are remapped per XCD) and C written once with coalesced stores.
 //   3. inverseBinMajor:  C[bin][i][j] -> planes, gathering runs of SLOTS
 //      consecutive j per bin, inverse transform, crop on store.
 //
 // Spectra are unpacked (N/2+1 rows) so the contraction is a plain complex GEMM.
-#include <stdlib.h>
-
 #include "common.h"
 #include "fft2d_core.h"
 #include "fft_regs.h"
@@ -162,28 +160,40 @@ struct GemmArgs {
   float invNorm;
 };
 
-template <int GJ, int GK>
-__global__ __launch_bounds__(kT, 2) void binGemm(GemmArgs g) {
-  constexpr int NA = GK * GI / 2 / kT;                 // float4 of A per lane per slice
-  constexpr int NB = (GK * GJ / 2 + kT - 1) / kT;      // float4 of B per lane per slice
-  constexpr int NQ = GJ / 32;  // 32-column MFMA sub-tiles per wave
-  __shared__ __align__(16) float2 As[2][GK][GI];
-  __shared__ __align__(16) float2 Bs[2][GK][GJ];
+// The k-slices go from HBM straight into LDS (global_load_lds, 16 bytes per lane,
+// no staging registers or LDS store instructions) through a ring of three slices:
+// slice s+2 is requested before slice s is multiplied, one barrier per slice.  A wave instruction moves 1 KiB: one k-row of A (128 complex)
+// or two k-rows of B (2 x 64 complex); LDS has exactly the HBM layout.  Requires
+// Kp % 8 == 0 with the padding rows zeroed; rows / columns beyond Ip / Jp are
+// clamped (they only feed accumulators that are never stored).
+constexpr int GJ2 = 64, GK2 = 8, ST = 3;
+
+__device__ __forceinline__ void loadToLds(const float2* src, float2* ldsWaveBase) {
+  __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
+                                   (__attribute__((address_space(3))) void*)ldsWaveBase, 16, 0, 0);
+}
+
+__global__ __launch_bounds__(kT, 2) void binGemmDirect(GemmArgs g) {
+  constexpr int NQ = GJ2 / 32;
+  __shared__ __align__(16) float2 As[ST][GK2][GI];
+  __shared__ __align__(16) float2 Bs[ST][GK2][GJ2];
   const int t = threadIdx.x;
   const int lane = t % 64, w = t / 64;
   const int r = lane % 32, h = lane / 32;
 
-  // consecutive logical ids on one XCD (workgroups are dealt round-robin to 8 XCDs)
   const int total = g.bins * g.IT * g.JT;
   const int per = (total + 7) / 8;
   const int logical = (blockIdx.x % 8) * per + blockIdx.x / 8;
   if (logical >= total) return;
   const int bin = logical / (g.IT * g.JT);
   const int rem = logical % (g.IT * g.JT);
-  const int i0 = (rem / g.JT) * GI, j0 = (rem % g.JT) * GJ;
+  const int i0 = (rem / g.JT) * GI, j0 = (rem % g.JT) * GJ2;
 
   const float2* Ab = g.A + (long)bin * g.Kp * g.Ip;
   const float2* Bb = g.B + (long)bin * g.Kp * g.Jp;
+  // per-lane source columns, clamped into the padded arrays
+  const int ia = min(i0 + 2 * lane, g.Ip - 2);
+  const int jb = min(j0 + 2 * (lane % 32), g.Jp - 2);
 
   floatx16 cre[NQ], cim[NQ];
 #pragma unroll
@@ -194,66 +204,49 @@ __global__ __launch_bounds__(kT, 2) void binGemm(GemmArgs g) {
       cim[q][v] = 0.f;
     }
 
-  // slice loads: A 8 x 128 complex = 512 float4 (2 per lane), B 8 x 64 = 256 float4 (1 per lane)
-  float4 ra[NA], rb[NB];
-  auto fetch = [&](int k0) {
-#pragma unroll
-    for (int u = 0; u < NA; ++u) {
-      const int idx = t + kT * u;
-      const int kk = idx / (GI / 2), ii = 2 * (idx % (GI / 2));
-      ra[u] = float4{0.f, 0.f, 0.f, 0.f};
-      if (k0 + kk < g.Kp && i0 + ii < g.Ip)
-        ra[u] = *reinterpret_cast<const float4*>(Ab + (long)(k0 + kk) * g.Ip + i0 + ii);
-    }
-#pragma unroll
-    for (int u = 0; u < NB; ++u) {
-      const int idx = t + kT * u;
-      const int kk = idx / (GJ / 2), jj = 2 * (idx % (GJ / 2));
-      rb[u] = float4{0.f, 0.f, 0.f, 0.f};
-      if (kk < GK && k0 + kk < g.Kp && j0 + jj < g.Jp)
-        rb[u] = *reinterpret_cast<const float4*>(Bb + (long)(k0 + kk) * g.Jp + j0 + jj);
-    }
-  };
-  auto stash = [&](int buf) {
-#pragma unroll
-    for (int u = 0; u < NA; ++u) {
-      const int idx = t + kT * u;
-      *reinterpret_cast<float4*>(&As[buf][idx / (GI / 2)][2 * (idx % (GI / 2))]) = ra[u];
-    }
-#pragma unroll
-    for (int u = 0; u < NB; ++u) {
-      const int idx = t + kT * u;
-      if (idx / (GJ / 2) < GK)
-        *reinterpret_cast<float4*>(&Bs[buf][idx / (GJ / 2)][2 * (idx % (GJ / 2))]) = rb[u];
-    }
+  // wave w moves rows 2w, 2w+1 of A and rows 2w, 2w+1 of B of a slice: 3 instructions
+  auto issue = [&](int sl) {
+    const int st = sl % ST;
+    const int k0 = sl * GK2;
+    loadToLds(Ab + (long)(k0 + 2 * w) * g.Ip + ia, &As[st][2 * w][0]);
+    loadToLds(Ab + (long)(k0 + 2 * w + 1) * g.Ip + ia, &As[st][2 * w + 1][0]);
+    loadToLds(Bb + (long)(k0 + 2 * w + h) * g.Jp + jb, &Bs[st][2 * w][0]);
   };
 
-  fetch(0);
-  stash(0);
-  __syncthreads();
-  const int slices = (g.Kp + GK - 1) / GK;
+  const int slices = g.Kp / GK2;
+  issue(0);
+  if (slices > 1) issue(1);
   for (int sl = 0; sl < slices; ++sl) {
-    const int cur = sl & 1;
-    if (sl + 1 < slices) fetch((sl + 1) * GK);
+    // this wave's loads of slice sl have landed once at most the 3 of slice sl+1 are pending
+    if (sl + 1 < slices)
+      __builtin_amdgcn_s_waitcnt(0x0F73);  // vmcnt(3)
+    else
+      __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+    __syncthreads();                       // ... and so have everybody else's; slice sl-1 is consumed
+    if (sl + 2 < slices) issue(sl + 2);
+    const int cur = sl % ST;
+    float2 av[GK2 / 2], bv[GK2 / 2][NQ];
 #pragma unroll
-    for (int s2 = 0; s2 < GK / 2; ++s2) {
-      const float2 a = As[cur][2 * s2 + h][32 * w + r];
+    for (int s2 = 0; s2 < GK2 / 2; ++s2) {
+      av[s2] = As[cur][2 * s2 + h][32 * w + r];
+#pragma unroll
+      for (int q = 0; q < NQ; ++q) bv[s2][q] = Bs[cur][2 * s2 + h][32 * q + r];
+    }
+#pragma unroll
+    for (int s2 = 0; s2 < GK2 / 2; ++s2) {
+      const float2 a = av[s2];
       const float nar = -a.x;
 #pragma unroll
       for (int q = 0; q < NQ; ++q) {
-        const float2 b = Bs[cur][2 * s2 + h][32 * q + r];
-        // a * conj(b): re = ar*br + ai*bi, im = ai*br - ar*bi
+        const float2 b = bv[s2][q];
         cre[q] = __builtin_amdgcn_mfma_f32_32x32x2f32(a.x, b.x, cre[q], 0, 0, 0);
         cim[q] = __builtin_amdgcn_mfma_f32_32x32x2f32(a.y, b.x, cim[q], 0, 0, 0);
         cre[q] = __builtin_amdgcn_mfma_f32_32x32x2f32(a.y, b.y, cre[q], 0, 0, 0);
         cim[q] = __builtin_amdgcn_mfma_f32_32x32x2f32(nar, b.y, cim[q], 0, 0, 0);
       }
     }
-    if (sl + 1 < slices) stash(cur ^ 1);
-    __syncthreads();
   }
 
-  // register v of lane (r, h) holds row 8*(v/4) + 4*h + v%4 and column r of a sub-tile
   float2* Cb = g.C + (long)bin * g.I * g.Jp;
 #pragma unroll
   for (int q = 0; q < NQ; ++q) {
@@ -272,7 +265,7 @@ inline int roundUp(int a, int b) { return (a + b - 1) / b * b; }
 template <int N>
 size_t workspaceFloat2(int B, int Cin, int Cout) {
   const int SL = BMCfg<N>::SLOTS, bins = BMCfg<N>::BINS;
-  const int Ip = roundUp(B, SL), Jp = roundUp(Cout, SL), Kp = roundUp(Cin, 2);
+  const int Ip = roundUp(B, SL), Jp = roundUp(Cout, SL), Kp = roundUp(Cin, 8);
   return (size_t)bins * ((size_t)Kp * Ip + (size_t)Kp * Jp + (size_t)B * Jp);
 }
 
@@ -281,7 +274,7 @@ int runFprop(const PlaneSet& in, const PlaneSet& wt, const PlaneSet& out, int B,
              float2* ws, hipStream_t s) {
   using C = BMCfg<N>;
   const int SL = C::SLOTS, bins = C::BINS;
-  const int Ip = roundUp(B, SL), Jp = roundUp(Cout, SL), Kp = roundUp(Cin, 2);
+  const int Ip = roundUp(B, SL), Jp = roundUp(Cout, SL), Kp = roundUp(Cin, 8);
   float2* SA = ws;
   float2* SB = SA + (size_t)bins * Kp * Ip;
   float2* SC = SB + (size_t)bins * Kp * Jp;
@@ -299,15 +292,8 @@ int runFprop(const PlaneSet& in, const PlaneSet& wt, const PlaneSet& out, int B,
   g.Kp = Kp;
   g.IT = ceilDiv(B, GI);
   g.invNorm = 1.0f / (float)(N * N);
-  static const int gjEnv = getenv("FBFFT_GEMM_GJ") ? atoi(getenv("FBFFT_GEMM_GJ")) : 64;
-  static const int gkEnv = getenv("FBFFT_GEMM_GK") ? atoi(getenv("FBFFT_GEMM_GK")) : 8;
-  g.JT = ceilDiv(Jp, gjEnv == 32 ? 32 : 64);
-  const dim3 grid(roundUp(bins * g.IT * g.JT, 8));
-  if (gjEnv == 32 && gkEnv == 16) binGemm<32, 16><<<grid, dim3(kT), 0, s>>>(g);
-  else if (gjEnv == 32) binGemm<32, 8><<<grid, dim3(kT), 0, s>>>(g);
-  else if (gkEnv == 16) binGemm<64, 16><<<grid, dim3(kT), 0, s>>>(g);
-  else if (gkEnv == 4) binGemm<64, 4><<<grid, dim3(kT), 0, s>>>(g);
-  else binGemm<64, 8><<<grid, dim3(kT), 0, s>>>(g);
+  g.JT = ceilDiv(Jp, GJ2);
+  binGemmDirect<<<dim3(roundUp(bins * g.IT * g.JT, 8)), dim3(kT), 0, s>>>(g);
   inverseBinMajor<N><<<dim3(Jp / SL, B), dim3(kT), 0, s>>>(SC, B, Jp, out);
   return launchStatus();
 }
