@@ -126,6 +126,28 @@ def conv_extras(F, synth, torch, dev, extra):
     extra["fft_conv_configs3_ms_per_iter"] = round(t * 1e3, 4)
     extra["fft_conv_configs3_direct_equiv_TFLOPs"] = round(41.6e9 / t / 1e12, 1)
     extra["fft_conv_configs3_fp32_peak_direct_ms"] = round(41.6e9 / 157.3e12 * 1e3, 4)
+    # the other two passes of the same layer
+    g = synth.normal((128, 192, 23, 23), seed=32, device=dev)
+    gi, gw = torch.empty_like(x), torch.empty_like(w)
+    vg, vgi, vgw = F.view(g), F.view(gi), F.view(gw)
+    ws2 = torch.empty(max(F.conv_workspace(1, 128, 64, 192, 32), F.conv_workspace(2, 128, 64, 192, 32)),
+                      dtype=torch.uint8, device=dev)
+    wsp2, wsb2 = ctypes.c_void_p(ws2.data_ptr()), ws2.numel()
+
+    def bprop():
+        if L.fbfft_conv_bprop(ctypes.byref(vg), ctypes.byref(vw), ctypes.byref(vgi), 32, wsp2, wsb2,
+                              stream) != 0:
+            raise RuntimeError("fbfft_conv_bprop failed")
+
+    def accgrad():
+        if L.fbfft_conv_accgrad(ctypes.byref(vx), ctypes.byref(vg), ctypes.byref(vgw), 32,
+                                ctypes.c_float(1.0), 0, wsp2, wsb2, stream) != 0:
+            raise RuntimeError("fbfft_conv_accgrad failed")
+    _, t = timed(bprop, 50, 5, torch)
+    extra["fft_conv_configs3_bprop_ms_per_iter"] = round(t * 1e3, 4)
+    _, t = timed(accgrad, 50, 5, torch)
+    extra["fft_conv_configs3_accgrad_ms_per_iter"] = round(t * 1e3, 4)
+    del g, gi, gw, ws2
     A = synth.normal((128, 64, 17, 32, 2), seed=30, device=dev)
     Bm = synth.normal((192, 64, 17, 32, 2), seed=31, device=dev)
     C = torch.empty((128, 192, 17, 32, 2), device=dev)
@@ -139,13 +161,7 @@ def conv_extras(F, synth, torch, dev, extra):
     x4 = synth.uniform((16, 32, 256, 256), seed=40, device=dev)
     w4 = synth.normal((32, 32, 9, 9), seed=41, std=0.05, device=dev)
     o4 = torch.empty((16, 32, 248, 248), device=dev)
-    iv, ov = [], []
-    for y0 in range(0, 248, 24):
-        for x0 in range(0, 248, 24):
-            iv.append((y0, x0, min(32, 256 - y0), min(32, 256 - x0), 0, 0))
-            ov.append((y0, x0, min(24, 248 - y0), min(24, 248 - x0), 0, 0))
-    ins, n = F.make_tiles(x4, iv)
-    outs, _ = F.make_tiles(o4, ov)
+    ins, outs, n = F.make_tile_grid(x4, o4, 9, 9, 32)   # 11 x 11 tiles of stride 24
     vw4 = F.view(w4)
 
     def tiled():

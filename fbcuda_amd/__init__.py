@@ -46,8 +46,9 @@ _lib = None
 # every symbol include/fbfft_amd.h declares
 EXPORTS = (
     "fbfft_r2c_1d", "fbfft_c2r_1d", "fbfft_r2c_2d", "fbfft_c2c_2d_pass2", "fbfft_c2r_2d",
-    "fbfft_c2c_2d_inverse_pass1", "fbfft_transpose_mm", "fbfft_iterated_conv",
-    "fbfft_conv_fprop_workspace", "fbfft_conv_fprop", "fbfft_error_string",
+    "fbfft_c2c_2d_inverse_pass1", "fbfft_transpose_mm", "fbfft_iterated_conv", "fbfft_make_tiles",
+    "fbfft_conv_workspace", "fbfft_conv_fprop_workspace", "fbfft_conv_fprop", "fbfft_conv_bprop",
+    "fbfft_conv_accgrad", "fbfft_error_string",
     "fbfft_twiddle_table",
 )
 
@@ -73,9 +74,17 @@ def lib():
                                          ctypes.c_float, vp]
         L.fbfft_iterated_conv.argtypes = [ctypes.c_int, vp, vp, tp, ctypes.c_int, ctypes.c_float,
                                           ctypes.c_int, ctypes.c_size_t, vp]
+        L.fbfft_make_tiles.argtypes = [tp, tp, ctypes.c_int, ctypes.c_int, ctypes.c_int, vp, vp,
+                                       ctypes.c_size_t]
+        L.fbfft_make_tiles.restype = ctypes.c_size_t
         L.fbfft_conv_fprop_workspace.argtypes = [ctypes.c_int] * 4
         L.fbfft_conv_fprop_workspace.restype = ctypes.c_size_t
         L.fbfft_conv_fprop.argtypes = [tp, tp, tp, ctypes.c_int, vp, ctypes.c_size_t, vp]
+        L.fbfft_conv_workspace.argtypes = [ctypes.c_int] * 5
+        L.fbfft_conv_workspace.restype = ctypes.c_size_t
+        L.fbfft_conv_bprop.argtypes = [tp, tp, tp, ctypes.c_int, vp, ctypes.c_size_t, vp]
+        L.fbfft_conv_accgrad.argtypes = [tp, tp, tp, ctypes.c_int, ctypes.c_float, ctypes.c_int, vp,
+                                         ctypes.c_size_t, vp]
         L.fbfft_error_string.argtypes = [ctypes.c_int]
         L.fbfft_error_string.restype = ctypes.c_char_p
         L.fbfft_twiddle_table.argtypes = [ctypes.POINTER(ctypes.c_float)]
@@ -185,6 +194,23 @@ def make_tiles(t, windows):
     return host.to(t.device), len(windows)
 
 
+def make_tile_grid(input, output, kH, kW, fftSize):
+    """The overlap tiling of a whole layer (fbfft_make_tiles): device descriptor
+    arrays (ins, outs) for `input` [B][Cin][H][W] and `output` [B][Cout][H-kH+1][W-kW+1],
+    and the tile count.  Raises on unsupported arguments."""
+    import torch
+    vi, vo = view(input), view(output)
+    n = lib().fbfft_make_tiles(vi, vo, kH, kW, fftSize, None, None, 0)
+    if n == 0:
+        raise ValueError("fbfft_make_tiles: unsupported arguments")
+    a, b = (Tile * n)(), (Tile * n)()
+    got = lib().fbfft_make_tiles(vi, vo, kH, kW, fftSize, ctypes.cast(a, ctypes.c_void_p),
+                                 ctypes.cast(b, ctypes.c_void_p), n)
+    assert got == n
+    up = lambda arr: torch.frombuffer(bytearray(bytes(arr)), dtype=torch.uint8).to(input.device)
+    return up(a), up(b), n
+
+
 def FFTIteratedConvolution(fftSize, ins, outs, weight, pass_, scale, batchSize, numTiles,
                            stream=None):
     """detail::FFTIteratedConvolution<fftSize> (fbfft/FFTIteratedConvolution.cuh:624-755).
@@ -210,3 +236,26 @@ def conv_fprop(input, weight, output, fftSize, workspace, stream=None):
     return lib().fbfft_conv_fprop(view(input), view(weight), view(output), fftSize,
                                   ctypes.c_void_p(workspace.data_ptr()),
                                   workspace.numel() * workspace.element_size(), _stream(stream))
+
+
+def conv_workspace(pass_, batch, cin, cout, fftSize):
+    """Workspace bytes of pass 0 (conv_fprop), 1 (conv_bprop) or 2 (conv_accgrad)."""
+    return lib().fbfft_conv_workspace(int(pass_), batch, cin, cout, fftSize)
+
+
+def conv_bprop(gradOutput, weight, gradInput, fftSize, workspace, stream=None):
+    """updateGradInput: gradInput[b][c] = sum_f fullconv(gradOutput[b][f], weight[f][c])."""
+    _on_gpu(gradOutput, weight, gradInput, workspace)
+    return lib().fbfft_conv_bprop(view(gradOutput), view(weight), view(gradInput), fftSize,
+                                  ctypes.c_void_p(workspace.data_ptr()),
+                                  workspace.numel() * workspace.element_size(), _stream(stream))
+
+
+def conv_accgrad(input, gradOutput, gradWeight, fftSize, workspace, scale=1.0, accumulate=False,
+                 stream=None):
+    """accGradParameters: gradWeight[f][c] (+)= scale * sum_b corr(input[b][c], gradOutput[b][f])."""
+    _on_gpu(input, gradOutput, gradWeight, workspace)
+    return lib().fbfft_conv_accgrad(view(input), view(gradOutput), view(gradWeight), fftSize,
+                                    ctypes.c_float(scale), int(bool(accumulate)),
+                                    ctypes.c_void_p(workspace.data_ptr()),
+                                    workspace.numel() * workspace.element_size(), _stream(stream))

@@ -3,6 +3,8 @@
 #include <string.h>
 
 #include "common.h"
+
+#include <algorithm>
 #include "fft_regs.h"
 
 using namespace fbfft_amd;
@@ -173,19 +175,17 @@ extern "C" int fbfft_transpose_mm(const fbfft_tensor* A, const fbfft_tensor* B,
                            conjA != 0, conjB != 0, accumulate != 0, invNorm, stream);
 }
 
-extern "C" size_t fbfft_conv_fprop_workspace(int batch, int cin, int cout, int fftSize) {
-  if (batch <= 0 || cin <= 0 || cout <= 0) return 0;
-  if (!(fftSize == 8 || fftSize == 16 || fftSize == 32)) return 0;
-  return convFpropWorkspaceBytes(fftSize, batch, cin, cout);
-}
+namespace {
 
-extern "C" int fbfft_conv_fprop(const fbfft_tensor* input, const fbfft_tensor* weight,
-                                const fbfft_tensor* output, int fftSize, void* workspace,
-                                size_t workspaceBytes, fbfft_stream_t stream) {
+bool convSizeOk(int N) { return N == 8 || N == 16 || N == 32; }
+
+// Shapes of one convolution layer: input [B][Cin][H][W], weight [Cout][Cin][kH][kW],
+// output [B][Cout][H-kH+1][W-kW+1], H, W <= N.
+int checkConvShapes(const fbfft_tensor* input, const fbfft_tensor* weight,
+                    const fbfft_tensor* output, int N) {
   if (!okTensor(input, 4) || !okTensor(weight, 4) || !okTensor(output, 4))
     return FBFFT_UNSUPPORTED_DIMENSION;
-  const int N = fftSize;
-  if (!(N == 8 || N == 16 || N == 32)) return FBFFT_UNSUPPORTED_SIZE;
+  if (!convSizeOk(N)) return FBFFT_UNSUPPORTED_SIZE;
   const int B = input->size[0], Cin = input->size[1], H = input->size[2], W = input->size[3];
   const int Cout = weight->size[0], kH = weight->size[2], kW = weight->size[3];
   if (weight->size[1] != Cin || output->size[0] != B || output->size[1] != Cout)
@@ -193,13 +193,62 @@ extern "C" int fbfft_conv_fprop(const fbfft_tensor* input, const fbfft_tensor* w
   if (H > N || W > N || kH > H || kW > W) return FBFFT_UNSUPPORTED_SIZE;
   if (output->size[2] != H - kH + 1 || output->size[3] != W - kW + 1)
     return FBFFT_UNSUPPORTED_DIMENSION;
+  return FBFFT_SUCCESS;
+}
+
+int convPass(int pass, const fbfft_tensor* input, const fbfft_tensor* weight,
+             const fbfft_tensor* output, int N, float scale, bool accumulate, void* workspace,
+             size_t workspaceBytes, fbfft_stream_t stream) {
+  const int rc = checkConvShapes(input, weight, output, N);
+  if (rc != FBFFT_SUCCESS) return rc;
   if (empty(input) || empty(weight) || empty(output)) return FBFFT_SUCCESS;
   if (!workspace || !aligned(workspace, 256) ||
-      workspaceBytes < fbfft_conv_fprop_workspace(B, Cin, Cout, N))
+      workspaceBytes < fbfft_conv_workspace(pass, input->size[0], input->size[1], weight->size[0], N))
     return FBFFT_UNSUPPORTED_DIMENSION;
-  return launchConvFprop(N, input->data, input->stride, input->size, weight->data, weight->stride,
-                         weight->size, output->data, output->stride, output->size, workspace,
-                         stream);
+  const fbfft_tensor *x, *y, *out;
+  if (pass == 0) {
+    x = input, y = weight, out = output;
+  } else if (pass == 1) {
+    x = output, y = weight, out = input;
+  } else {
+    x = input, y = output, out = weight;
+  }
+  return launchConvPass(pass, N, x->data, x->stride, x->size, y->data, y->stride, y->size,
+                        out->data, out->stride, out->size, scale, accumulate, workspace, stream);
+}
+
+}  // namespace
+
+extern "C" size_t fbfft_conv_workspace(int pass, int batch, int cin, int cout, int fftSize) {
+  if (pass < 0 || pass > 2 || batch <= 0 || cin <= 0 || cout <= 0) return 0;
+  if (!convSizeOk(fftSize)) return 0;
+  return convWorkspaceBytes(pass, fftSize, batch, cin, cout);
+}
+
+extern "C" size_t fbfft_conv_fprop_workspace(int batch, int cin, int cout, int fftSize) {
+  return fbfft_conv_workspace(0, batch, cin, cout, fftSize);
+}
+
+extern "C" int fbfft_conv_fprop(const fbfft_tensor* input, const fbfft_tensor* weight,
+                                const fbfft_tensor* output, int fftSize, void* workspace,
+                                size_t workspaceBytes, fbfft_stream_t stream) {
+  return convPass(0, input, weight, output, fftSize, 1.0f, false, workspace, workspaceBytes,
+                  stream);
+}
+
+extern "C" int fbfft_conv_bprop(const fbfft_tensor* gradOutput, const fbfft_tensor* weight,
+                                const fbfft_tensor* gradInput, int fftSize, void* workspace,
+                                size_t workspaceBytes, fbfft_stream_t stream) {
+  return convPass(1, gradInput, weight, gradOutput, fftSize, 1.0f, false, workspace,
+                  workspaceBytes, stream);
+}
+
+extern "C" int fbfft_conv_accgrad(const fbfft_tensor* input, const fbfft_tensor* gradOutput,
+                                  const fbfft_tensor* gradWeight, int fftSize, float scale,
+                                  int accumulate, void* workspace, size_t workspaceBytes,
+                                  fbfft_stream_t stream) {
+  return convPass(2, input, gradWeight, gradOutput, fftSize, scale, accumulate != 0, workspace,
+                  workspaceBytes, stream);
 }
 
 extern "C" int fbfft_c2c_2d_pass2(const fbfft_tensor* src, const fbfft_tensor* dst,
@@ -230,6 +279,45 @@ extern "C" int fbfft_c2c_2d_inverse_pass1(const fbfft_tensor* src, const fbfft_t
   return launchTwoPass(N, 2, src->data, src->stride[0], src->stride[1], src->stride[2], dst->data,
                        dst->stride[0], dst->stride[1], dst->stride[2], src->size[0], 0, 0, 0, 0,
                        stream);
+}
+
+extern "C" size_t fbfft_make_tiles(const fbfft_tensor* input, const fbfft_tensor* output, int kH,
+                                   int kW, int fftSize, fbfft_tile* ins, fbfft_tile* outs,
+                                   size_t capacity) {
+  if (!okTensor(input, 4) || !okTensor(output, 4)) return 0;
+  const int N = fftSize;
+  if (!(N == 8 || N == 16 || N == 32) || kH < 1 || kW < 1 || kH > N || kW > N) return 0;
+  const int H = input->size[2], W = input->size[3];
+  const int oH = H - kH + 1, oW = W - kW + 1;
+  if (oH < 1 || oW < 1 || output->size[2] != oH || output->size[3] != oW) return 0;
+  if (output->size[0] != input->size[0]) return 0;
+  const int stepY = N - kH + 1, stepX = N - kW + 1;
+  const size_t ny = (size_t)ceilDiv(oH, stepY), nx = (size_t)ceilDiv(oW, stepX);
+  if (!ins || !outs) return ny * nx;
+  size_t n = 0;
+  for (int y0 = 0; y0 < oH; y0 += stepY) {
+    for (int x0 = 0; x0 < oW; x0 += stepX, ++n) {
+      if (n >= capacity) continue;
+      fbfft_tile& ti = ins[n];
+      fbfft_tile& to = outs[n];
+      ti.padL = ti.padU = to.padL = to.padU = 0;
+      ti.data = input->data + (size_t)y0 * input->stride[2] + (size_t)x0 * input->stride[3];
+      to.data = output->data + (size_t)y0 * output->stride[2] + (size_t)x0 * output->stride[3];
+      for (int d = 0; d < 4; ++d) {
+        ti.stride[d] = input->stride[d];
+        to.stride[d] = output->stride[d];
+      }
+      ti.size[0] = input->size[0];
+      ti.size[1] = input->size[1];
+      ti.size[2] = std::min(N, H - y0);
+      ti.size[3] = std::min(N, W - x0);
+      to.size[0] = output->size[0];
+      to.size[1] = output->size[1];
+      to.size[2] = std::min(stepY, oH - y0);
+      to.size[3] = std::min(stepX, oW - x0);
+    }
+  }
+  return n;
 }
 
 extern "C" int fbfft_iterated_conv(int fftSize, const fbfft_tile* ins, const fbfft_tile* outs,

@@ -61,9 +61,11 @@ int launchIteratedConv(int N, const fbfft_tile* ins, const fbfft_tile* outs, flo
 int launchTwoPass(int N, int mode, float* src, long s0, long s1, long s2, float* dst, long d0,
                   long d1, long d2, int B, int h, int w, int padL, int padU, hipStream_t s);
 
-size_t convFpropWorkspaceBytes(int N, int B, int Cin, int Cout);
-int launchConvFprop(int N, float* in, const int* inStride, const int* inSize, float* wt,
-                    const int* wtStride, const int* wtSize, float* out, const int* outStride,
-                    const int* outSize, void* workspace, hipStream_t s);
+// pass 0 / 1 / 2 = forward, input gradient, weight gradient (x, y, out as in conv_pipeline.hip)
+size_t convWorkspaceBytes(int pass, int N, int B, int Cin, int Cout);
+int launchConvPass(int pass, int N, float* x, const int* xStride, const int* xSize, float* y,
+                   const int* yStride, const int* ySize, float* out, const int* outStride,
+                   const int* outSize, float scale, bool accumulate, void* workspace,
+                   hipStream_t s);
 
 }  // namespace fbfft_amd

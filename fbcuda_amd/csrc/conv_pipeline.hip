@@ -1,5 +1,7 @@
-// FFT convolution forward pass (valid cross-correlation) as three kernels that
-// hand spectra to each other in a layout chosen for the matrix cores.
+// The three passes of an FFT convolution layer (valid cross-correlation forward,
+// its gradient with respect to the input, its gradient with respect to the
+// weights), each as three kernels that hand spectra to each other in a layout
+// chosen for the matrix cores.
 //
 // The reference's external callers run fbfft2D -> transposeMM -> fbifft2D on
 // plane-major spectra [plane][bin] (MM-inl.cuh:188-196), which makes the
@@ -20,9 +22,18 @@
 //      consecutive j per bin, inverse transform, crop on store.
 //
 // Spectra are unpacked (N/2+1 rows) so the contraction is a plain complex GEMM.
+//
+// All three passes are the same product P[i][j] = sum_k X[i][k] * op(Y[j][k]) with
+// the roles of MM-inl.cuh:188-196: forward (i, j, k) = (image, output plane, input
+// plane), op = conj; input gradient (image, input plane, output plane), op =
+// identity; weight gradient (input plane, output plane, image), op = conj.  The
+// kernels always compute sum_k A * conj(B); the forward transforms store a
+// spectrum conjugated where the pass needs it.
 #include "common.h"
 #include "fft2d_core.h"
 #include "fft_regs.h"
+
+#include <utility>
 
 namespace fbfft_amd {
 namespace {
@@ -49,7 +60,8 @@ struct PlaneSet {
 
 // ---- 1. planes -> S[bin][k][row] ----
 template <int N>
-__global__ __launch_bounds__(kT) void forwardBinMajor(PlaneSet ps, float2* S, int Rp, int Kp) {
+__global__ __launch_bounds__(kT) void forwardBinMajor(PlaneSet ps, float2* S, int Rp, int Kp,
+                                                      float imSign) {
   using C = BMCfg<N>;
   constexpr int H = C::H, T = C::T, SLOTS = C::SLOTS, RS = C::RS, PSZ = C::PSZ;
   __shared__ __align__(16) c32 lds[SLOTS * PSZ];
@@ -89,13 +101,15 @@ __global__ __launch_bounds__(kT) void forwardBinMajor(PlaneSet ps, float2* S, in
     } else {
       v = src[r * RS + x];
     }
+    v.y *= imSign;
     dst[bin * binStride] = v;
   }
 }
 
 // ---- 3. C[bin][i][j] -> planes (i, j), cropped ----
-template <int N>
-__global__ __launch_bounds__(kT) void inverseBinMajor(const float2* Cs, int I, int Jp, PlaneSet out) {
+template <int N, bool ACC>
+__global__ __launch_bounds__(kT) void inverseBinMajor(const float2* Cs, int I, int Jp, PlaneSet out,
+                                                      float scale) {
   using C = BMCfg<N>;
   constexpr int H = C::H, T = C::T, SLOTS = C::SLOTS, RS = C::RS, PSZ = C::PSZ;
   __shared__ __align__(16) c32 lds[SLOTS * PSZ];
@@ -144,8 +158,8 @@ __global__ __launch_bounds__(kT) void inverseBinMajor(const float2* Cs, int I, i
   columnPassInverse<N>(plane, l, z0, z1);
   const int j = j0 + s;
   if (j < out.K)  // out.K: number of valid output planes along j
-    storeColumnsWindow<N>(out.base + (long)i * out.sRow + (long)j * out.sK, out.sy, out.sx, out.h,
-                          out.w, 0, 0, l, z0, z1, 1.0f);
+    storeColumnsWindow<N, ACC>(out.base + (long)i * out.sRow + (long)j * out.sK, out.sy, out.sx,
+                               out.h, out.w, 0, 0, l, z0, z1, scale);
 }
 
 // ---- 2. batched complex GEMM, bin-major ----
@@ -262,65 +276,120 @@ __global__ __launch_bounds__(kT, 2) void binGemmDirect(GemmArgs g) {
 
 inline int roundUp(int a, int b) { return (a + b - 1) / b * b; }
 
-template <int N>
-size_t workspaceFloat2(int B, int Cin, int Cout) {
-  const int SL = BMCfg<N>::SLOTS, bins = BMCfg<N>::BINS;
-  const int Ip = roundUp(B, SL), Jp = roundUp(Cout, SL), Kp = roundUp(Cin, 8);
-  return (size_t)bins * ((size_t)Kp * Ip + (size_t)Kp * Jp + (size_t)B * Jp);
+// Which operand takes the 128-wide side of the GEMM tile: the assignment with
+// fewer padded tile elements.
+inline bool swapRoles(int I, int J) {
+  return (long)roundUp(J, GI) * roundUp(I, GJ2) < (long)roundUp(I, GI) * roundUp(J, GJ2);
 }
 
 template <int N>
-int runFprop(const PlaneSet& in, const PlaneSet& wt, const PlaneSet& out, int B, int Cin, int Cout,
-             float2* ws, hipStream_t s) {
+size_t workspaceFloat2(int I, int J, int K) {
+  if (swapRoles(I, J)) std::swap(I, J);
+  const int SL = BMCfg<N>::SLOTS, bins = BMCfg<N>::BINS;
+  const int Ip = roundUp(I, SL), Jp = roundUp(J, SL), Kp = roundUp(K, 8);
+  return (size_t)bins * ((size_t)Kp * Ip + (size_t)Kp * Jp + (size_t)I * Jp);
+}
+
+// P[i][j] = scale * sum_k X[i][k] * op(Y[j][k]) for planes x(i,k), y(j,k) -> planes out(i,j);
+// each PlaneSet names its first index "row" and its second "k".
+template <int N>
+int runPipeline(PlaneSet x, PlaneSet y, PlaneSet out, bool conjY, float scale, bool accumulate,
+                float2* ws, hipStream_t s) {
   using C = BMCfg<N>;
   const int SL = C::SLOTS, bins = C::BINS;
-  const int Ip = roundUp(B, SL), Jp = roundUp(Cout, SL), Kp = roundUp(Cin, 8);
+  float xSign = 1.0f, ySign = conjY ? 1.0f : -1.0f;
+  if (swapRoles(x.R, y.R)) {
+    // G[j][i] = sum_k op(Y[j]) * conj(conj X[i])
+    std::swap(x, y);
+    xSign = conjY ? -1.0f : 1.0f;
+    ySign = -1.0f;
+    std::swap(out.sRow, out.sK);
+  }
+  const int I = x.R, J = y.R, K = x.K;
+  out.R = I;
+  out.K = J;
+  const int Ip = roundUp(I, SL), Jp = roundUp(J, SL), Kp = roundUp(K, 8);
   float2* SA = ws;
   float2* SB = SA + (size_t)bins * Kp * Ip;
   float2* SC = SB + (size_t)bins * Kp * Jp;
 
-  forwardBinMajor<N><<<dim3(Ip / SL, Kp), dim3(kT), 0, s>>>(in, SA, Ip, Kp);
-  forwardBinMajor<N><<<dim3(Jp / SL, Kp), dim3(kT), 0, s>>>(wt, SB, Jp, Kp);
+  forwardBinMajor<N><<<dim3(Ip / SL, Kp), dim3(kT), 0, s>>>(x, SA, Ip, Kp, xSign);
+  forwardBinMajor<N><<<dim3(Jp / SL, Kp), dim3(kT), 0, s>>>(y, SB, Jp, Kp, ySign);
   GemmArgs g;
   g.A = SA;
   g.B = SB;
   g.C = SC;
   g.bins = bins;
-  g.I = B;
+  g.I = I;
   g.Ip = Ip;
   g.Jp = Jp;
   g.Kp = Kp;
-  g.IT = ceilDiv(B, GI);
-  g.invNorm = 1.0f / (float)(N * N);
+  g.IT = ceilDiv(I, GI);
   g.JT = ceilDiv(Jp, GJ2);
+  g.invNorm = 1.0f / (float)(N * N);
   binGemmDirect<<<dim3(roundUp(bins * g.IT * g.JT, 8)), dim3(kT), 0, s>>>(g);
-  inverseBinMajor<N><<<dim3(Jp / SL, B), dim3(kT), 0, s>>>(SC, B, Jp, out);
+  if (accumulate)
+    inverseBinMajor<N, true><<<dim3(Jp / SL, I), dim3(kT), 0, s>>>(SC, I, Jp, out, scale);
+  else
+    inverseBinMajor<N, false><<<dim3(Jp / SL, I), dim3(kT), 0, s>>>(SC, I, Jp, out, scale);
   return launchStatus();
+}
+
+PlaneSet planes(float* base, const int* stride, const int* size, int rowDim, int kDim) {
+  return PlaneSet{base, stride[rowDim], stride[kDim], stride[2], stride[3], size[2], size[3],
+                  size[rowDim], size[kDim]};
+}
+
+template <int N>
+int runPass(int pass, const PlaneSet& x, const PlaneSet& y, const PlaneSet& out, float scale,
+            bool accumulate, float2* ws, hipStream_t s) {
+  return runPipeline<N>(x, y, out, /*conjY=*/pass != 1, scale, accumulate, ws, s);
 }
 
 }  // namespace
 
-size_t convFpropWorkspaceBytes(int N, int B, int Cin, int Cout) {
-  size_t n = N == 8 ? workspaceFloat2<8>(B, Cin, Cout)
-                    : N == 16 ? workspaceFloat2<16>(B, Cin, Cout) : workspaceFloat2<32>(B, Cin, Cout);
+// (I, J, K) of a pass for batch B and Cin / Cout planes
+static void passDims(int pass, int B, int Cin, int Cout, int* I, int* J, int* K) {
+  if (pass == 0) { *I = B; *J = Cout; *K = Cin; }
+  else if (pass == 1) { *I = B; *J = Cin; *K = Cout; }
+  else { *I = Cin; *J = Cout; *K = B; }
+}
+
+size_t convWorkspaceBytes(int pass, int N, int B, int Cin, int Cout) {
+  int I, J, K;
+  passDims(pass, B, Cin, Cout, &I, &J, &K);
+  size_t n = N == 8 ? workspaceFloat2<8>(I, J, K)
+                    : N == 16 ? workspaceFloat2<16>(I, J, K) : workspaceFloat2<32>(I, J, K);
   return n * sizeof(float2);
 }
 
-// input [B][Cin][H][W], weight [Cout][Cin][kH][kW], output [B][Cout][oH][oW]; strides in floats
-int launchConvFprop(int N, float* in, const int* inStride, const int* inSize, float* wt,
-                    const int* wtStride, const int* wtSize, float* out, const int* outStride,
-                    const int* outSize, void* workspace, hipStream_t s) {
-  const int B = inSize[0], Cin = inSize[1], Cout = wtSize[0];
-  PlaneSet pin{in, inStride[0], inStride[1], inStride[2], inStride[3], inSize[2], inSize[3], B, Cin};
-  PlaneSet pwt{wt, wtStride[0], wtStride[1], wtStride[2], wtStride[3], wtSize[2], wtSize[3], Cout, Cin};
-  // for the output, "row" is the image and "k" the output plane
-  PlaneSet pout{out, outStride[0], outStride[1], outStride[2], outStride[3], outSize[2], outSize[3],
-                B, Cout};
+// pass 0: x = input [B][Cin][H][W], y = weight [Cout][Cin][kH][kW], out = output [B][Cout][oH][oW]
+// pass 1: x = gradOutput [B][Cout][oH][oW], y = weight, out = gradInput [B][Cin][H][W]
+// pass 2: x = input, y = gradOutput, out = gradWeight [Cout][Cin][kH][kW]
+// strides in floats
+int launchConvPass(int pass, int N, float* x, const int* xStride, const int* xSize, float* y,
+                   const int* yStride, const int* ySize, float* out, const int* outStride,
+                   const int* outSize, float scale, bool accumulate, void* workspace,
+                   hipStream_t s) {
+  PlaneSet px, py, po;
+  if (pass == 0) {
+    px = planes(x, xStride, xSize, 0, 1);
+    py = planes(y, yStride, ySize, 0, 1);
+    po = planes(out, outStride, outSize, 0, 1);
+  } else if (pass == 1) {
+    px = planes(x, xStride, xSize, 0, 1);
+    py = planes(y, yStride, ySize, 1, 0);
+    po = planes(out, outStride, outSize, 0, 1);
+  } else {
+    px = planes(x, xStride, xSize, 1, 0);
+    py = planes(y, yStride, ySize, 1, 0);
+    po = planes(out, outStride, outSize, 1, 0);
+  }
   float2* ws = static_cast<float2*>(workspace);
   switch (N) {
-    case 8: return runFprop<8>(pin, pwt, pout, B, Cin, Cout, ws, s);
-    case 16: return runFprop<16>(pin, pwt, pout, B, Cin, Cout, ws, s);
-    case 32: return runFprop<32>(pin, pwt, pout, B, Cin, Cout, ws, s);
+    case 8: return runPass<8>(pass, px, py, po, scale, accumulate, ws, s);
+    case 16: return runPass<16>(pass, px, py, po, scale, accumulate, ws, s);
+    case 32: return runPass<32>(pass, px, py, po, scale, accumulate, ws, s);
   }
   return FBFFT_UNSUPPORTED_SIZE;
 }

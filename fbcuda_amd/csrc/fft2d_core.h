@@ -105,14 +105,20 @@ __device__ __forceinline__ void columnPassInverse(const c32* plane, int l, c32 (
 }
 
 // Two columns of results through a bounds-checked strided view (crop on store).
-template <int N>
+// ACC adds the scaled result to what the view holds instead of replacing it.
+template <int N, bool ACC = false>
 __device__ __forceinline__ void storeColumnsWindow(float* dst, int sy, int sx, int h, int w, int padL,
                                                    int padU, int l, const c32 (&z0)[N / 2],
                                                    const c32 (&z1)[N / 2], float scale) {
   const int x0 = 2 * l, x1 = 2 * l + 1;
   auto put = [&](int y, int x, float v) {
-    if (inWindow(y, x, padU, padL, h, w))
-      dst[(size_t)(y - padU) * sy + (size_t)(x - padL) * sx] = v * scale;
+    if (inWindow(y, x, padU, padL, h, w)) {
+      float* p = dst + (size_t)(y - padU) * sy + (size_t)(x - padL) * sx;
+      if constexpr (ACC)
+        *p += v * scale;
+      else
+        *p = v * scale;
+    }
   };
   staticFor<N / 2>([&](auto jj) {
     constexpr int j = decltype(jj)::value;

@@ -130,18 +130,57 @@ int fbfft_iterated_conv(int fftSize, const fbfft_tile* ins, const fbfft_tile* ou
                         const fbfft_tensor* weight, int pass, float scale, int batchSize,
                         size_t numTiles, fbfft_stream_t stream);
 
-/* Bytes of device workspace fbfft_conv_fprop needs for the given problem. */
+/* Host-side builder of the tile descriptors FFTIteratedConvolution consumes; the
+ * reference leaves this to its external caller (fbfft/FFTIteratedConvolution.cuh:
+ * 71-88 declares the descriptor, :113-114 consumes ins[tile] / outs[tile]).
+ * input is [B][Cin][H][W] and output [B][Cout][H-kH+1][W-kW+1] (device tensors;
+ * only their addresses and strides are used).  Tile t covers the output window
+ * whose origin advances by fftSize-kH+1 rows / fftSize-kW+1 columns, clipped at
+ * the edges, and the fftSize x fftSize (clipped) input window at the same
+ * origin; padL = padU = 0.  Row-major over (tileY, tileX).  Writes at most
+ * capacity descriptors into the HOST arrays ins / outs, which the caller then
+ * copies to the device, and returns the number of tiles of the grid; with
+ * ins == NULL or outs == NULL it only returns that number.  0 = unsupported
+ * arguments.  The same descriptor arrays serve all three passes. */
+size_t fbfft_make_tiles(const fbfft_tensor* input, const fbfft_tensor* output, int kH, int kW,
+                        int fftSize, fbfft_tile* ins, fbfft_tile* outs, size_t capacity);
+
+/* FFT convolution layer on the split path: the FFT -> transposeMM -> IFFT
+ * sequences that the reference's external callers compose from the primitives
+ * above, one entry point per pass of the role table at MM-inl.cuh:188-196.
+ * Shapes throughout: input / gradInput [B][Cin][H][W], weight / gradWeight
+ * [Cout][Cin][kH][kW], output / gradOutput [B][Cout][H-kH+1][W-kW+1], with
+ * H, W <= fftSize in {8,16,32}.  Valid cross-correlation, no kernel flip.
+ * workspace: device memory of at least fbfft_conv_workspace() bytes for that
+ * pass, 256-byte aligned; its contents need not survive between calls. */
+
+/* Bytes of workspace for pass 0 (fprop), 1 (bprop) or 2 (accgrad): the values of
+ * FFTConvolutionPassFFI (fbfft/FFTIteratedConvolution.cuh:616-622).  0 when the
+ * arguments are not supported. */
+size_t fbfft_conv_workspace(int pass, int batch, int cin, int cout, int fftSize);
+
+/* Same as fbfft_conv_workspace(0, ...). */
 size_t fbfft_conv_fprop_workspace(int batch, int cin, int cout, int fftSize);
 
-/* FFT convolution forward pass: the FFT -> transposeMM<false,true> -> IFFT
- * sequence that the reference's external callers compose from the primitives
- * above (MM-inl.cuh:188-196 role table).  Valid cross-correlation (no kernel
- * flip): input [B][Cin][H][W], weight [Cout][Cin][kH][kW], H, W <= fftSize in
- * {8,16,32}, output [B][Cout][H-kH+1][W-kW+1].  workspace: device memory of at
- * least fbfft_conv_fprop_workspace() bytes, 256-byte aligned. */
+/* updateOutput: transposeMM<false, true> role (MM-inl.cuh:194).
+ * output[b][f] = sum_c corr(input[b][c], weight[f][c]). */
 int fbfft_conv_fprop(const fbfft_tensor* input, const fbfft_tensor* weight,
                      const fbfft_tensor* output, int fftSize, void* workspace,
                      size_t workspaceBytes, fbfft_stream_t stream);
+
+/* updateGradInput: transposeMM<false, false> role (MM-inl.cuh:196).
+ * gradInput[b][c] = sum_f fullconv(gradOutput[b][f], weight[f][c]). */
+int fbfft_conv_bprop(const fbfft_tensor* gradOutput, const fbfft_tensor* weight,
+                     const fbfft_tensor* gradInput, int fftSize, void* workspace,
+                     size_t workspaceBytes, fbfft_stream_t stream);
+
+/* accGradParameters: transposeMM<true, false> role (MM-inl.cuh:195).
+ * gradWeight[f][c] = (accumulate ? gradWeight[f][c] : 0)
+ *                    + scale * sum_b corr(input[b][c], gradOutput[b][f]). */
+int fbfft_conv_accgrad(const fbfft_tensor* input, const fbfft_tensor* gradOutput,
+                       const fbfft_tensor* gradWeight, int fftSize, float scale,
+                       int accumulate, void* workspace, size_t workspaceBytes,
+                       fbfft_stream_t stream);
 
 /* Human-readable name of an fbfft_error. */
 const char* fbfft_error_string(int code);

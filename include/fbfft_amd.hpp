@@ -230,6 +230,17 @@ bool FFTIteratedConvolution(TiledDeviceTensor<float, 4>* ins, TiledDeviceTensor<
                              batchSize, numTiles, s) == 1;
 }
 
+// Host-side tile grid for FFTIteratedConvolution<FFTSize>: fills ins / outs (host
+// arrays of capacity descriptors) and returns the tile count; see fbfft_make_tiles.
+template <int FFTSize>
+size_t makeTiles(const DeviceTensor<float, 4>& input, const DeviceTensor<float, 4>& output, int kH,
+                 int kW, TiledDeviceTensor<float, 4>* ins, TiledDeviceTensor<float, 4>* outs,
+                 size_t capacity) {
+  fbfft_tensor i = fbfft_amd_detail::describe(input), o = fbfft_amd_detail::describe(output);
+  return fbfft_make_tiles(&i, &o, kH, kW, FFTSize, reinterpret_cast<fbfft_tile*>(ins),
+                          reinterpret_cast<fbfft_tile*>(outs), capacity);
+}
+
 }  // namespace detail
 }  // namespace fbfft
 
@@ -240,6 +251,46 @@ void transposeMM(DeviceTensor<float, Dim>& A, DeviceTensor<float, Dim>& B,
                c = fbfft_amd_detail::describe(C);
   fbfft_transpose_mm(&a, &b, &c, ConjugateTransposeA, ConjugateTransposeB, Accumulate, invNorm, s);
 }
+
+// The three passes of a convolution layer on the split FFT -> transposeMM -> IFFT
+// path, which the reference's external callers compose themselves
+// (MM-inl.cuh:188-196).  workspace: device memory of fftConvolutionWorkspace bytes.
+namespace fbfft {
+
+inline size_t fftConvolutionWorkspace(detail::FFTConvolutionPassFFI pass, int batch, int cin,
+                                      int cout, int fftSize) {
+  return fbfft_conv_workspace(pass.pass, batch, cin, cout, fftSize);
+}
+
+inline FBFFTParameters::ErrorCode fftConvolutionUpdateOutput(
+    DeviceTensor<float, 4>& input, DeviceTensor<float, 4>& weight, DeviceTensor<float, 4>& output,
+    int fftSize, void* workspace, size_t workspaceBytes, fbfft_stream_t s = 0) {
+  fbfft_tensor i = fbfft_amd_detail::describe(input), w = fbfft_amd_detail::describe(weight),
+               o = fbfft_amd_detail::describe(output);
+  return amd_detail::code(fbfft_conv_fprop(&i, &w, &o, fftSize, workspace, workspaceBytes, s));
+}
+
+inline FBFFTParameters::ErrorCode fftConvolutionUpdateGradInput(
+    DeviceTensor<float, 4>& gradOutput, DeviceTensor<float, 4>& weight,
+    DeviceTensor<float, 4>& gradInput, int fftSize, void* workspace, size_t workspaceBytes,
+    fbfft_stream_t s = 0) {
+  fbfft_tensor g = fbfft_amd_detail::describe(gradOutput), w = fbfft_amd_detail::describe(weight),
+               i = fbfft_amd_detail::describe(gradInput);
+  return amd_detail::code(fbfft_conv_bprop(&g, &w, &i, fftSize, workspace, workspaceBytes, s));
+}
+
+inline FBFFTParameters::ErrorCode fftConvolutionAccGradParameters(
+    DeviceTensor<float, 4>& input, DeviceTensor<float, 4>& gradOutput,
+    DeviceTensor<float, 4>& gradWeight, int fftSize, float scale, bool accumulate, void* workspace,
+    size_t workspaceBytes, fbfft_stream_t s = 0) {
+  fbfft_tensor i = fbfft_amd_detail::describe(input), g = fbfft_amd_detail::describe(gradOutput),
+               w = fbfft_amd_detail::describe(gradWeight);
+  return amd_detail::code(fbfft_conv_accgrad(&i, &g, &w, fftSize, scale, accumulate, workspace,
+                                             workspaceBytes, s));
+}
+
+}  // namespace fbfft
+
 
 } }  // namespace facebook::cuda
 

@@ -91,3 +91,66 @@ def test_cpp_facade_compiles_against_reference_include_paths():
     subprocess.check_call(["make", "-C", os.path.join(ROOT, "tests", "cpp"), "-B"],
                           stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL)
     assert os.path.exists(os.path.join(ROOT, "tests", "cpp", "facade_check"))
+
+
+def _fake_tensor(shape, base=0x10000000):
+    """fbfft_tensor over memory that is never touched: the tile builder only does
+    address arithmetic."""
+    t = F.Tensor()
+    t.data = base
+    t.dim = len(shape)
+    stride = 1
+    for i in reversed(range(len(shape))):
+        t.size[i] = shape[i]
+        t.stride[i] = stride
+        stride *= shape[i]
+    return t
+
+
+@pytest.mark.parametrize("H,W,kH,kW,N", [
+    (256, 256, 9, 9, 32),    # configs[4]: 11 x 11 tiles, the last 16 wide in, 8 wide out
+    (32, 32, 5, 5, 32), (40, 56, 9, 3, 32), (14, 17, 3, 3, 8), (30, 25, 5, 1, 16), (9, 9, 1, 1, 8)])
+def test_make_tiles_grid(H, W, kH, kW, N):
+    Bn, Cin, Cout = 3, 2, 5
+    oH, oW = H - kH + 1, W - kW + 1
+    ti, to = _fake_tensor((Bn, Cin, H, W)), _fake_tensor((Bn, Cout, oH, oW), 0x20000000)
+    L = F.lib()
+    n = L.fbfft_make_tiles(ti, to, kH, kW, N, None, None, 0)
+    sy, sx = N - kH + 1, N - kW + 1
+    ys, xs = list(range(0, oH, sy)), list(range(0, oW, sx))
+    assert n == len(ys) * len(xs)
+    a, b = (F.Tile * n)(), (F.Tile * n)()
+    assert L.fbfft_make_tiles(ti, to, kH, kW, N, ctypes.cast(a, ctypes.c_void_p),
+                              ctypes.cast(b, ctypes.c_void_p), n) == n
+    covered = np.zeros((oH, oW), np.int32)
+    for t, (y0, x0) in enumerate((y, x) for y in ys for x in xs):
+        assert (a[t].padL, a[t].padU, b[t].padL, b[t].padU) == (0, 0, 0, 0)
+        assert a[t].data == 0x10000000 + 4 * (y0 * W + x0)
+        assert b[t].data == 0x20000000 + 4 * (y0 * oW + x0)
+        assert list(a[t].stride) == [Cin * H * W, H * W, W, 1]
+        assert list(b[t].stride) == [Cout * oH * oW, oH * oW, oW, 1]
+        assert list(a[t].size) == [Bn, Cin, min(N, H - y0), min(N, W - x0)]
+        assert list(b[t].size) == [Bn, Cout, min(sy, oH - y0), min(sx, oW - x0)]
+        # the input window holds every sample the output window needs
+        assert a[t].size[2] >= b[t].size[2] + kH - 1 and a[t].size[3] >= b[t].size[3] + kW - 1
+        covered[y0:y0 + b[t].size[2], x0:x0 + b[t].size[3]] += 1
+    assert (covered == 1).all()   # output windows partition the output plane
+    if (H, N) == (256, 32):
+        assert n == 121 and a[n - 1].size[2] == 16 and b[n - 1].size[2] == 8
+
+
+def test_make_tiles_capacity_and_rejects():
+    ti, to = _fake_tensor((1, 1, 40, 40)), _fake_tensor((1, 1, 36, 36))
+    L = F.lib()
+    a, b = (F.Tile * 2)(), (F.Tile * 2)()
+    pa, pb = ctypes.cast(a, ctypes.c_void_p), ctypes.cast(b, ctypes.c_void_p)
+    assert L.fbfft_make_tiles(ti, to, 5, 5, 16, pa, pb, 2) == 9    # 3 x 3 grid, two written
+    assert a[1].data == 0x10000000 + 4 * 12
+    assert L.fbfft_make_tiles(ti, to, 5, 5, 64, None, None, 0) == 0    # FFT size
+    assert L.fbfft_make_tiles(ti, to, 3, 3, 16, None, None, 0) == 0    # output shape mismatch
+    assert L.fbfft_make_tiles(ti, to, 5, 17, 16, None, None, 0) == 0   # kernel wider than the FFT
+    assert F.lib().fbfft_conv_workspace(0, 128, 64, 192, 32) == \
+        F.lib().fbfft_conv_fprop_workspace(128, 64, 192, 32) > 0
+    for p in (0, 1, 2):
+        assert F.lib().fbfft_conv_workspace(p, 4, 5, 6, 16) % 8 == 0
+    assert F.lib().fbfft_conv_workspace(0, 4, 5, 6, 64) == 0

@@ -146,3 +146,21 @@ def test_config4_forward(oracle):
     oh = out.cpu().numpy()
     got = oh[coords[:, 0], coords[:, 1], coords[:, 2], coords[:, 3]]
     assert rel(got, want) < TOL_CONV
+
+
+def test_library_tile_grid_matches_reference_tiling(oracle):
+    """fbfft_make_tiles builds the descriptors that tiles_for spells out; the
+    forward pass over them equals fp64 direct correlation."""
+    N, k, H, W, Nb, Cin, Cout = 16, 5, 37, 30, 2, 3, 4
+    d = dev()
+    x = synth.uniform((Nb, Cin, H, W), seed=40, device=d)
+    w = synth.normal((Cout, Cin, k, k), seed=41, std=0.05, device=d)
+    out = torch.full((Nb, Cout, H - k + 1, W - k + 1), float("nan"), device=d)
+    ins, outs, n = F.make_tile_grid(x, out, k, k, N)
+    iv, ov = tiles_for(H, W, k, N)
+    ins2, n2 = F.make_tiles(x, iv)
+    outs2, _ = F.make_tiles(out, ov)
+    assert n == n2 and bool((ins == ins2).all()) and bool((outs == outs2).all())
+    assert F.FFTIteratedConvolution(N, ins, outs, w, F.FFT_UpdateOutput, 1.0, Nb, n)
+    torch.cuda.synchronize()
+    assert rel(out.cpu().numpy(), oracle.corr2d_valid(x.cpu().numpy(), w.cpu().numpy())) < TOL_CONV

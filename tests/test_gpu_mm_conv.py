@@ -130,3 +130,77 @@ def test_conv_fprop_config3(oracle):
     assert rel(got, want) < TOL_CONV
     full = oracle.corr2d_valid(xh[[0, 127]], wh[[0, 191]])
     assert rel(oh[[0, 127]][:, [0, 191]], full) < TOL_CONV
+
+
+SHAPES = [(8, 8, 8, 3, 2, 3, 4), (16, 13, 16, 5, 3, 5, 7), (32, 27, 27, 5, 4, 8, 6),
+          (32, 32, 30, 1, 2, 2, 2), (32, 20, 31, 7, 5, 150, 9), (16, 16, 16, 3, 70, 3, 140)]
+
+
+def workspace(pass_, Bn, Cin, Cout, N):
+    return torch.empty(F.conv_workspace(pass_, Bn, Cin, Cout, N), dtype=torch.uint8, device=dev())
+
+
+@pytest.mark.parametrize("N,H,W,k,Bn,Cin,Cout", SHAPES)
+def test_conv_bprop(oracle, N, H, W, k, Bn, Cin, Cout):
+    """updateGradInput against the fp64 gradient of the direct correlation."""
+    go = synth.normal((Bn, Cout, H - k + 1, W - k + 1), seed=32).numpy()
+    w = synth.normal((Cout, Cin, k, k), seed=31, std=0.02).numpy()
+    d = dev()
+    gi = torch.full((Bn, Cin, H, W), float("nan"), device=d)
+    rc = F.conv_bprop(torch.from_numpy(go).to(d), torch.from_numpy(w).to(d), gi, N,
+                      workspace(1, Bn, Cin, Cout, N))
+    torch.cuda.synchronize()
+    assert rc == F.Success
+    assert rel(gi.cpu().numpy(), oracle.corr2d_grad_input(go, w, H, W)) < TOL_CONV
+
+
+@pytest.mark.parametrize("accumulate", [False, True])
+@pytest.mark.parametrize("N,H,W,k,Bn,Cin,Cout", SHAPES)
+def test_conv_accgrad(oracle, N, H, W, k, Bn, Cin, Cout, accumulate):
+    """accGradParameters against the fp64 gradient; with accumulate the old
+    gradient stays and the new one is added with weight `scale`."""
+    x = synth.normal((Bn, Cin, H, W), seed=30).numpy()
+    go = synth.normal((Bn, Cout, H - k + 1, W - k + 1), seed=32).numpy()
+    d = dev()
+    gw0 = synth.normal((Cout, Cin, k, k), seed=34).numpy()
+    gw = torch.from_numpy(gw0.copy()).to(d) if accumulate else \
+        torch.full((Cout, Cin, k, k), float("nan"), device=d)
+    scale = 0.25
+    rc = F.conv_accgrad(torch.from_numpy(x).to(d), torch.from_numpy(go).to(d), gw, N,
+                        workspace(2, Bn, Cin, Cout, N), scale=scale, accumulate=accumulate)
+    torch.cuda.synchronize()
+    assert rc == F.Success
+    want = scale * oracle.corr2d_grad_weight(x, go, k, k) + (gw0 if accumulate else 0.0)
+    assert rel(gw.cpu().numpy(), want) < TOL_CONV
+
+
+def test_conv_passes_are_adjoint():
+    """configs[3] shapes: <conv(x, w), g> = <x, bprop(g, w)> = <w, accgrad(x, g)> ties the three
+    passes together at full size without a CPU reference."""
+    d = dev()
+    x = synth.normal((128, 64, 27, 27), seed=30, device=d)
+    w = synth.normal((192, 64, 5, 5), seed=31, std=0.02, device=d)
+    g = synth.normal((128, 192, 23, 23), seed=32, device=d)
+    out, gi, gw = torch.empty_like(g), torch.empty_like(x), torch.empty_like(w)
+    assert F.conv_fprop(x, w, out, 32, workspace(0, 128, 64, 192, 32)) == F.Success
+    assert F.conv_bprop(g, w, gi, 32, workspace(1, 128, 64, 192, 32)) == F.Success
+    assert F.conv_accgrad(x, g, gw, 32, workspace(2, 128, 64, 192, 32)) == F.Success
+    torch.cuda.synchronize()
+    a = float((out.double() * g.double()).sum())
+    b = float((x.double() * gi.double()).sum())
+    c = float((w.double() * gw.double()).sum())
+    assert abs(a - b) <= 1e-4 * abs(a) and abs(a - c) <= 1e-4 * abs(a)
+
+
+def test_conv_pass_argument_checks():
+    d = dev()
+    x = torch.zeros(2, 3, 16, 16, device=d)
+    w = torch.zeros(4, 3, 3, 3, device=d)
+    o = torch.zeros(2, 4, 14, 14, device=d)
+    ws = workspace(1, 2, 3, 4, 16)
+    assert F.conv_bprop(o, w, x, 16, ws) == F.Success
+    assert F.conv_bprop(o, w, x, 64, ws) == F.UnsupportedSize
+    assert F.conv_bprop(o[:, :3], w, x, 16, ws) == F.UnsupportedDimension
+    assert F.conv_accgrad(x, o, w[:, :, :2], 16, ws) == F.UnsupportedDimension
+    assert F.conv_bprop(o, w, x, 16, ws[:16]) == F.UnsupportedDimension
+    assert F.conv_workspace(3, 2, 3, 4, 16) == 0
