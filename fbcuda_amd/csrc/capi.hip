@@ -111,7 +111,8 @@ int fbfft_r2c_2d(const fbfft_tensor* real, const fbfft_tensor* cplx, int padL, i
   const int s1 = cplx->size[1], s2 = cplx->size[2];
   int N = 0;
   bool scratchForm = false;
-  if ((s2 == 8 || s2 == 16 || s2 == 32 || s2 == 64 || s2 == 128) && s1 == s2 / 2 + 1) {
+  if ((s2 == 2 || s2 == 4 || s2 == 8 || s2 == 16 || s2 == 32 || s2 == 64 || s2 == 128) &&
+      s1 == s2 / 2 + 1) {
     N = s2;
   } else if ((s1 == 64 || s1 == 128) && s2 == s1 / 2 + 1) {
     N = s1;
@@ -123,6 +124,7 @@ int fbfft_r2c_2d(const fbfft_tensor* real, const fbfft_tensor* cplx, int padL, i
     return FBFFT_UNSUPPORTED_SIZE;
   if (!okCplx(cplx)) return FBFFT_UNSUPPORTED_DIMENSION;
   if (empty(real) || empty(cplx)) return FBFFT_SUCCESS;
+  if (N < 8) return launchFft2dTinyForward(N, realView3(real), cplxView4(cplx), padL, padU, stream);
   if (N <= 32) return launchFft2dSmallForward(N, realView3(real), cplxView4(cplx), padL, padU, stream);
   if (!scratchForm)
     return launchFft2dLargeForward(N, realView3(real), cplxView4(cplx), padL, padU, stream);
@@ -137,13 +139,15 @@ int fbfft_c2r_2d(const fbfft_tensor* cplx, const fbfft_tensor* real, int padL, i
   if (cplx->size[3] != 2) return FBFFT_UNSUPPORTED_DIMENSION;
   if (real->size[0] != cplx->size[0]) return FBFFT_UNSUPPORTED_DIMENSION;
   const int s1 = cplx->size[1], N = cplx->size[2];
-  if (!(N == 8 || N == 16 || N == 32 || N == 64 || N == 128)) return FBFFT_UNSUPPORTED_SIZE;
+  if (!(N == 2 || N == 4 || N == 8 || N == 16 || N == 32 || N == 64 || N == 128))
+    return FBFFT_UNSUPPORTED_SIZE;
   const bool half = (s1 == N / 2 + 1);
   const bool full = (N >= 64 && s1 == N);
   if (!half && !full) return FBFFT_UNSUPPORTED_SIZE;
   if (padL < 0 || padU < 0) return FBFFT_UNSUPPORTED_SIZE;
   if (!okCplx(cplx)) return FBFFT_UNSUPPORTED_DIMENSION;
   if (empty(real) || empty(cplx)) return FBFFT_SUCCESS;
+  if (N < 8) return launchFft2dTinyInverse(N, cplxView4(cplx), realView3(real), padL, padU, stream);
   if (N <= 32) return launchFft2dSmallInverse(N, cplxView4(cplx), realView3(real), padL, padU, stream);
   if (half) return launchFft2dLargeInverse(N, cplxView4(cplx), realView3(real), padL, padU, stream);
   return launchTwoPass(N, 3, cplx->data, cplx->stride[0], cplx->stride[1], cplx->stride[2],

@@ -41,6 +41,11 @@ int launchFft2dSmallForward(int N, const RealView& real, const CplxView& cplx, i
 int launchFft2dSmallInverse(int N, const CplxView& cplx, const RealView& real, int padL, int padU,
                             hipStream_t s);
 
+int launchFft2dTinyForward(int N, const RealView& real, const CplxView& cplx, int padL, int padU,
+                           hipStream_t s);
+int launchFft2dTinyInverse(int N, const CplxView& cplx, const RealView& real, int padL, int padU,
+                           hipStream_t s);
+
 int launchFft2dLargeForward(int N, const RealView& real, const CplxView& cplx, int padL, int padU,
                             hipStream_t s);
 int launchFft2dLargeInverse(int N, const CplxView& cplx, const RealView& real, int padL, int padU,

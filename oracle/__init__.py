@@ -170,8 +170,8 @@ def idft1d_c2r(cplx):
 
 
 def layout_of(N):
-    """0: [ky half][kx] (N <= 32), 1: [kx half][ky] (N >= 64)."""
-    return 0 if N <= 32 else 1
+    """0: [ky half][kx] (N in 8, 16, 32), 1: [kx half][ky] (N in 2, 4 and N >= 64)."""
+    return 0 if 8 <= N <= 32 else 1
 
 
 def dft2d_r2c(real, N, padL=0, padU=0, layout=None):

@@ -391,6 +391,53 @@ void fbifft2dLargePair(const float* in0, const float* in1, int N, int h, int w,
   }
 }
 
+// ---------------------------------------------------------------------------
+// 2D, N in {2, 4}: the warp kernel that the entry point falls through to for
+// sizes the register kernels do not cover (FBFFT2D-inl.cuh:124-222, dispatch
+// :571-615).  Planes b and b+1 ride as the real and imaginary part of one
+// complex row transform (load2DR2C, :45-69), the two spectra are separated with
+// the Hermitian split (:171-183), transposed, and the first N/2+1 columns are
+// transformed again; store2D (:71-85) writes cplx[b][kx][ky], the same layout as
+// N >= 64.  The inverse for these sizes (FBIFFT2D-inl.cuh:188-247, dispatch
+// :684-712) is the one-kernel form of fbifft2dLargePair above with the same
+// plane pairing b, b + ceil(B/2).
+// ---------------------------------------------------------------------------
+
+void fbfft2dWarpPair(const float* p0, const float* p1, int h, int w, int N, int padL, int padU,
+                     float* out0, float* out1) {
+  const int nc = N / 2 + 1;
+  std::vector<cf> A((size_t)N * N), Bv((size_t)N * N), v(N);  // [y][kx]
+  for (int y = 0; y < N; ++y) {
+    for (int x = 0; x < N; ++x) {
+      if (inBounds2(y, x, padU, padL, h, w)) {
+        const size_t i = (size_t)(y - padU) * w + x - padL;
+        v[x] = mk(p0[i], p1 ? p1[i] : 0.0f);
+      } else {
+        v[x] = mk(0.0f, 0.0f);
+      }
+    }
+    difStages(v.data(), 1, N, true);
+    bitReverse(v.data(), 1, N);
+    for (int x = 0; x < N; ++x) {
+      const cf me = v[x], other = v[(N - x) % N];
+      A[(size_t)y * N + x] = mk(0.5f * (me.re + other.re), 0.5f * (me.im - other.im));
+      Bv[(size_t)y * N + x] = mk(0.5f * (me.im + other.im), 0.5f * (-me.re + other.re));
+    }
+  }
+  for (int which = 0; which < 2; ++which) {
+    float* out = which == 0 ? out0 : out1;
+    if (!out) continue;
+    const std::vector<cf>& src = which == 0 ? A : Bv;
+    cf* o = reinterpret_cast<cf*>(out);
+    for (int kx = 0; kx < nc; ++kx) {
+      for (int y = 0; y < N; ++y) v[y] = src[(size_t)y * N + kx];
+      difStages(v.data(), 1, N, true);
+      bitReverse(v.data(), 1, N);
+      for (int ky = 0; ky < N; ++ky) o[(size_t)kx * N + ky] = v[ky];
+    }
+  }
+}
+
 // TiledDeviceTensor<float,4> (FFTIteratedConvolution.cuh:71-88) with the
 // DeviceTensor member order data, stride, size (DeviceTensor.cuh:237-245).
 struct TileDesc {
@@ -475,11 +522,20 @@ int orc_fbifft1d(const float* cplx, int B, int N, int padL, float* real) {
 
 // fbfft2D<1> (FBFFT2D-inl.cuh:450-669): real [B][h][w] (contiguous) placed at
 // (padU, padL) of a zero N x N plane -> cplx [B][N/2+1][N][2].
-// N <= 32: cplx[b][ky][kx]; N >= 64: cplx[b][kx][ky].
+// N in {8,16,32}: cplx[b][ky][kx]; N in {2,4} and N >= 64: cplx[b][kx][ky].
 int orc_fbfft2d(const float* real, int B, int h, int w, int N, int padL, int padU,
                 float* cplx) {
-  if (!(N == 8 || N == 16 || N == 32 || N == 64 || N == 128)) return 1;
+  if (!(N == 2 || N == 4 || N == 8 || N == 16 || N == 32 || N == 64 || N == 128)) return 1;
   const size_t inPlane = (size_t)h * w, outPlane = (size_t)(N / 2 + 1) * N * 2;
+  if (N < 8) {
+#pragma omp parallel for schedule(static)
+    for (int b = 0; b < B; b += 2) {
+      const bool two = b + 1 < B;
+      fbfft2dWarpPair(real + b * inPlane, two ? real + (b + 1) * inPlane : nullptr, h, w, N, padL,
+                      padU, cplx + b * outPlane, two ? cplx + (b + 1) * outPlane : nullptr);
+    }
+    return 0;
+  }
 #pragma omp parallel for schedule(static)
   for (int b = 0; b < B; ++b) {
     if (N <= 32)
@@ -494,9 +550,9 @@ int orc_fbfft2d(const float* real, int B, int h, int w, int N, int padL, int pad
 // real [B][h][w], gain N*N, cropped to the (padU, padL) window.
 int orc_fbifft2d(const float* cplx, int B, int N, int h, int w, int padL, int padU,
                  float* real) {
-  if (!(N == 8 || N == 16 || N == 32 || N == 64 || N == 128)) return 1;
+  if (!(N == 2 || N == 4 || N == 8 || N == 16 || N == 32 || N == 64 || N == 128)) return 1;
   const size_t outPlane = (size_t)h * w, inPlane = (size_t)(N / 2 + 1) * N * 2;
-  if (N <= 32) {
+  if (N >= 8 && N <= 32) {
 #pragma omp parallel for schedule(static)
     for (int b = 0; b < B; ++b)
       fbifft2dSmallPlane(cplx + b * inPlane, N, h, w, padL, padU, real + b * outPlane);

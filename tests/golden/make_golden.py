@@ -5,8 +5,8 @@ reference holds no vectors for this path) in float64, stored in the reference's
 output layouts:
 
   1D            cplx[b][k]          k  = 0..N/2
-  2D, N <= 32   cplx[b][ky][kx]     ky = 0..N/2   (fft2(X)[:N/2+1, :])
-  2D, N >= 64   cplx[b][kx][ky]     kx = 0..N/2   (rfft2(X) transposed)
+  2D, N = 8, 16, 32      cplx[b][ky][kx]     ky = 0..N/2   (fft2(X)[:N/2+1, :])
+  2D, N = 2, 4, 64, 128  cplx[b][kx][ky]     kx = 0..N/2   (rfft2(X) transposed)
 
 Run from the repository root:  python tests/golden/make_golden.py
 """
@@ -21,13 +21,14 @@ for N in (8, 32, 256):
     out["x1d_%d" % N] = x
     out["f1d_%d" % N] = np.fft.rfft(x.astype(np.float64), axis=1)
 for N, h, w, padL, padU in ((8, 8, 8, 0, 0), (16, 11, 9, 2, 3), (32, 27, 27, 0, 0),
-                            (32, 5, 5, 0, 0), (64, 64, 64, 0, 0), (128, 100, 90, 5, 7)):
+                            (32, 5, 5, 0, 0), (64, 64, 64, 0, 0), (128, 100, 90, 5, 7),
+                            (4, 4, 4, 0, 0), (4, 3, 3, 1, 0), (2, 2, 2, 0, 0)):
     nb = 2 if N <= 32 else 1
     x = rng.standard_normal((nb, h, w)).astype(np.float32)
     X = np.zeros((nb, N, N))
     X[:, padU:padU + h, padL:padL + w] = x
     F = np.fft.fft2(X)
-    if N >= 64:
+    if N >= 64 or N < 8:
         F = np.transpose(F, (0, 2, 1))
     key = "%d_%d_%d_%d_%d" % (N, h, w, padL, padU)
     out["x2d_" + key] = x

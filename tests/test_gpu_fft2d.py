@@ -152,3 +152,33 @@ def test_two_groups_per_wave_tail(oracle, N, B):
     pick = [0, 1, B // 2, B - 130, B - 5, B - 4, B - 3, B - 2, B - 1]
     _, want = oracle.fbfft2d(x[pick].cpu().numpy(), N)
     assert rel(spec[pick].cpu().numpy(), want) < TOL_FFT
+
+
+@pytest.mark.parametrize("N", [2, 4])
+@pytest.mark.parametrize("B", [1, 2, 5, 1000])
+def test_warp_kernel_sizes(oracle, N, B):
+    """N = 2 and 4 (the reference's plane-pairing warp kernel, fbfft/FBFFT2D-inl.cuh:611-612):
+    transposed [kx half][ky] layout, odd batches, windows and padding."""
+    for h, w, padL, padU in [(N, N, 0, 0), (N - 1, N, 0, 0), (N - 1, N - 1, 1, 1)]:
+        x = synth.normal((B, h, w), seed=100 + N + B).numpy()
+        rc, got = fft2d(x, N, padL, padU)
+        assert rc == F.Success
+        _, want32 = oracle.fbfft2d(x, N, padL, padU)
+        assert rel(got, want32) < TOL_FFT
+        assert rel(got, oracle.dft2d_r2c(x, N, padL, padU)) < TOL_FFT
+        rc, back = ifft2d(want32, h, w, padL, padU)
+        assert rc == F.Success
+        _, back32 = oracle.fbifft2d(want32, h, w, padL, padU)
+        assert rel(back, back32) < TOL_FFT
+        assert rel(back, N * N * x.astype(np.float64)) < TOL_FFT
+    # strided views on both sides
+    x = synth.normal((B, N, N), seed=7).numpy()
+    big = torch.zeros((B, N + 1, N + 3), device=dev())
+    real = big[:, 1:, 2:N + 2]
+    real.copy_(torch.from_numpy(x))
+    wide = torch.full((B, N // 2 + 2, N + 1, 2), float("nan"), device=dev())
+    spec = wide[:, 1:, :N, :]
+    assert F.fbfft2D(real, spec) == F.Success
+    torch.cuda.synchronize()
+    assert rel(spec.cpu().numpy(), oracle.dft2d_r2c(x, N)) < TOL_FFT
+    assert bool(torch.isnan(wide[:, 0]).all()) and bool(torch.isnan(wide[:, :, N]).all())

@@ -27,7 +27,7 @@ def embed(x, N, padL, padU):
 
 def spec2d(X, N):
     F = np.fft.fft2(X)
-    if N >= 64:
+    if N >= 64 or N < 8:
         F = np.transpose(F, (0, 2, 1))
     return F[:, :N // 2 + 1, :]
 
@@ -174,8 +174,36 @@ def test_2d_vs_numpy_roundtrip_invariants(oracle, N, case):
         assert rel(c(out), c(o0) * ph[None]) < TOL
 
 
+@pytest.mark.parametrize("N", [2, 4])
+@pytest.mark.parametrize("B", [1, 2, 5])
+def test_2d_warp_sizes(oracle, N, B):
+    """N = 2 and 4 go through the plane-pairing warp kernel and use the transposed
+    [kx half][ky] layout; an odd batch leaves the last plane unpaired."""
+    rng = np.random.default_rng(10 * N + B)
+    for h, w, padL, padU in [(N, N, 0, 0), (N - 1, N, 0, 0), (N - 1, N - 1, 1, 1)]:
+        x = rng.standard_normal((B, h, w)).astype(np.float32)
+        rc, out = oracle.fbfft2d(x, N, padL, padU)
+        assert rc == 0 and out.shape == (B, N // 2 + 1, N, 2)
+        X = embed(x, N, padL, padU)
+        assert rel(c(out), spec2d(X, N)) < TOL
+        assert rel(c(oracle.dft2d_r2c(x, N, padL, padU)), spec2d(X, N)) < TOL64
+        rc, back = oracle.fbifft2d(out, h, w, padL, padU)
+        assert rc == 0 and rel(back, N * N * x.astype(np.float64)) < TOL
+    # closed forms, literal: impulse at (y0, x0) = (1, N-1); out[kx][ky]
+    x = np.zeros((1, N, N), np.float32)
+    x[0, 1, N - 1] = 1.0
+    _, out = oracle.fbfft2d(x, N)
+    k = np.arange(N)
+    want = np.exp(-2j * np.pi * (k[None, :] * 1 + k[:, None] * (N - 1)) / N)[:N // 2 + 1]  # [kx][ky]
+    assert np.abs(c(out)[0] - want).max() < 1e-6
+    # an x-only ramp has energy only at ky = 0: tells [kx][ky] from [ky][kx]
+    ramp = np.tile(np.arange(N, dtype=np.float32), (N, 1))[None]
+    _, out = oracle.fbfft2d(ramp, N)
+    assert np.abs(c(out)[0][:, 1:]).max() < 1e-6 and abs(c(out)[0][1, 0]) > 1.0
+
+
 def test_2d_unsupported_sizes(oracle):
-    for N in (4, 12, 256):
+    for N in (1, 12, 256):
         rc, _ = oracle.fbfft2d(np.zeros((1, N, N), np.float32), N)
         assert rc == 1
 
