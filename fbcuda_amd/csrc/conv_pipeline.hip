@@ -47,7 +47,10 @@ struct BMCfg {
   static constexpr int T = N / 2;
   static constexpr int SLOTS = kT / T;                 // planes per workgroup
   static constexpr int RS = PlaneCfg<N>::RS;
-  static constexpr int PSZ = (H + 1) * RS + 2;         // plane stride in LDS (complex), 16-byte aligned
+  // plane stride in LDS (complex): 16-byte aligned, and 4 banks mod 32 so that the
+  // transposed accesses (16 or more planes at the same bin) spread over the banks
+  static constexpr int PSZ = (H + 1) * RS;
+  static_assert((2 * PSZ) % 32 == 4 && PSZ % 2 == 0, "plane stride");
   static constexpr int BINS = (H + 1) * N;
 };
 
@@ -85,25 +88,31 @@ __global__ __launch_bounds__(kT) void forwardBinMajor(PlaneSet ps, float2* S, in
   rowPassInPlace<N, true>(plane, l);
   __syncthreads();
 
-  // lanes: sp = t % SLOTS walks the run (consecutive rows), bq = t / SLOTS walks bins
+  // lanes: sp = t % SLOTS walks the run (consecutive rows), bq = t / SLOTS in [0, T)
+  // walks bins: lane (sp, bq) stores columns x = bq and bq + T of every spectral row,
+  // so LDS and HBM offsets are compile-time constants on top of one per-lane base.
   const int sp = t % SLOTS, bq = t / SLOTS;
-  const c32* src = lds + sp * PSZ;
-  float2* dst = S + (long)k * Rp + r0 + sp;
+  const c32* src = lds + sp * PSZ + bq;
   const long binStride = (long)Kp * Rp;
-#pragma unroll 2
-  for (int bin = bq; bin < C::BINS; bin += T) {
-    const int r = bin / N, x = bin % N;
-    c32 v;
-    if (r == 0 || r == H) {
-      c32 a = src[x], m = src[(N - x) & (N - 1)];
-      v = r == 0 ? c32{0.5f * (a.x + m.x), 0.5f * (a.y - m.y)}
-                 : c32{0.5f * (a.y + m.y), 0.5f * (m.x - a.x)};
-    } else {
-      v = src[r * RS + x];
-    }
+  float2* dst = S + (long)k * Rp + r0 + sp + bq * binStride;
+  auto put = [&](int bin, c32 v) __attribute__((always_inline)) {
     v.y *= imSign;
     dst[bin * binStride] = v;
-  }
+  };
+  // rows 0 and N/2 share packed row 0: F0[x] = (P[x] + conj P[N-x]) / 2,
+  // FH[x] = (P[x] - conj P[N-x]) / 2i
+  staticFor<2>([&](auto ee) {
+    constexpr int e = decltype(ee)::value;
+    const int x = bq + T * e;
+    const c32 a = src[T * e], m = lds[sp * PSZ + ((N - x) & (N - 1))];
+    put(T * e, c32{0.5f * (a.x + m.x), 0.5f * (a.y - m.y)});
+    put(H * N + T * e, c32{0.5f * (a.y + m.y), 0.5f * (m.x - a.x)});
+  });
+  staticFor<H - 1>([&](auto rr) {
+    constexpr int r = decltype(rr)::value + 1;
+    put(r * N, src[r * RS]);
+    put(r * N + T, src[r * RS + T]);
+  });
 }
 
 // ---- 3. C[bin][i][j] -> planes (i, j), cropped ----
@@ -132,9 +141,8 @@ __global__ __launch_bounds__(kT) void inverseBinMajor(const float2* Cs, int I, i
       in[u] = src[(bq + T * u) * binStride];
     });
     staticFor<PER>([&](auto uu) {
-      constexpr int u = decltype(uu)::value;
-      const int bin = bq + T * u;
-      dstp[(bin / N) * RS + bin % N] = in[u];
+      constexpr int u = decltype(uu)::value;  // bin = bq + T*u: row u/2, column bq + T*(u%2)
+      dstp[(u / 2) * RS + T * (u % 2) + bq] = in[u];
     });
   }
   __syncthreads();

@@ -29,20 +29,30 @@ __device__ __forceinline__ void ldsStore4(c32* p, c32 a, c32 b) {
 
 // Two columns of a real plane through a bounds-checked strided view:
 // z[j] = (X[2j][x], X[2j+1][x]) for x = 2l and 2l+1, zero outside the window
-// (the padding rule of MemoryAccess.cuh:19-25).
+// (the padding rule of MemoryAccess.cuh:19-25).  Every load is issued
+// unconditionally at an address clamped into the window and the value is zeroed
+// afterwards, so the 2N loads of a lane are all in flight together and no branch
+// separates them; the window must not be empty.  Row terms are wave-uniform.
 template <int N>
 __device__ __forceinline__ void loadColumnsWindow(const float* src, int sy, int sx, int h, int w,
                                                   int padL, int padU, int l, c32 (&z0)[N / 2],
                                                   c32 (&z1)[N / 2]) {
-  const int x0 = 2 * l, x1 = 2 * l + 1;
-  auto fetch = [&](int y, int x) {
-    return inWindow(y, x, padU, padL, h, w)
-               ? src[(size_t)(y - padU) * sy + (size_t)(x - padL) * sx] : 0.0f;
-  };
+  const int xa = 2 * l - padL, xb = xa + 1;
+  const bool va = (unsigned)xa < (unsigned)w, vb = (unsigned)xb < (unsigned)w;
+  const float* pa = src + (long)min(max(xa, 0), w - 1) * sx;
+  const float* pb = src + (long)min(max(xb, 0), w - 1) * sx;
+  float ra[N], rb[N];
+  staticFor<N>([&](auto yy) {
+    constexpr int y = decltype(yy)::value;
+    const long oy = (long)min(max(y - padU, 0), h - 1) * sy;
+    ra[y] = pa[oy];
+    rb[y] = pb[oy];
+  });
   staticFor<N / 2>([&](auto jj) {
     constexpr int j = decltype(jj)::value;
-    z0[j] = c32{fetch(2 * j, x0), fetch(2 * j + 1, x0)};
-    z1[j] = c32{fetch(2 * j, x1), fetch(2 * j + 1, x1)};
+    const bool v0 = (unsigned)(2 * j - padU) < (unsigned)h, v1 = (unsigned)(2 * j + 1 - padU) < (unsigned)h;
+    z0[j] = c32{v0 && va ? ra[2 * j] : 0.0f, v1 && va ? ra[2 * j + 1] : 0.0f};
+    z1[j] = c32{v0 && vb ? rb[2 * j] : 0.0f, v1 && vb ? rb[2 * j + 1] : 0.0f};
   });
 }
 
