@@ -195,10 +195,17 @@ __device__ __forceinline__ void loadToLds(const float2* src, float2* ldsWaveBase
                                    (__attribute__((address_space(3))) void*)ldsWaveBase, 16, 0, 0);
 }
 
-__global__ __launch_bounds__(kT, 2) void binGemmDirect(GemmArgs g) {
+struct GemmStage {
+  float2 A[GK2][GI];
+  float2 B[GK2][GJ2];
+};
+
+__global__ __launch_bounds__(kT, 4) void binGemmDirect(GemmArgs g) {
   constexpr int NQ = GJ2 / 32;
-  __shared__ __align__(16) float2 As[ST][GK2][GI];
-  __shared__ __align__(16) float2 Bs[ST][GK2][GJ2];
+  // three separate variables, not one array: the compiler tracks pending
+  // global->LDS loads per LDS variable, so reading one stage does not wait for the
+  // loads still in flight into the other two
+  __shared__ __align__(16) GemmStage stage0, stage1, stage2;
   const int t = threadIdx.x;
   const int lane = t % 64, w = t / 64;
   const int r = lane % 32, h = lane / 32;
@@ -226,33 +233,33 @@ __global__ __launch_bounds__(kT, 2) void binGemmDirect(GemmArgs g) {
       cim[q][v] = 0.f;
     }
 
+  const int slices = g.Kp / GK2;
   // wave w moves rows 2w, 2w+1 of A and rows 2w, 2w+1 of B of a slice: 3 instructions
-  auto issue = [&](int sl) {
-    const int st = sl % ST;
+  auto issue = [&](GemmStage& st, int sl) __attribute__((always_inline)) {
     const int k0 = sl * GK2;
-    loadToLds(Ab + (long)(k0 + 2 * w) * g.Ip + ia, &As[st][2 * w][0]);
-    loadToLds(Ab + (long)(k0 + 2 * w + 1) * g.Ip + ia, &As[st][2 * w + 1][0]);
-    loadToLds(Bb + (long)(k0 + 2 * w + h) * g.Jp + jb, &Bs[st][2 * w][0]);
+    loadToLds(Ab + (long)(k0 + 2 * w) * g.Ip + ia, &st.A[2 * w][0]);
+    loadToLds(Ab + (long)(k0 + 2 * w + 1) * g.Ip + ia, &st.A[2 * w + 1][0]);
+    loadToLds(Bb + (long)(k0 + 2 * w + h) * g.Jp + jb, &st.B[2 * w][0]);
   };
 
-  const int slices = g.Kp / GK2;
-  issue(0);
-  if (slices > 1) issue(1);
-  for (int sl = 0; sl < slices; ++sl) {
-    // this wave's loads of slice sl have landed once at most the 3 of slice sl+1 are pending
-    if (sl + 1 < slices)
-      __builtin_amdgcn_s_waitcnt(0x0F73);  // vmcnt(3)
-    else
-      __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
-    __syncthreads();                       // ... and so have everybody else's; slice sl-1 is consumed
-    if (sl + 2 < slices) issue(sl + 2);
-    const int cur = sl % ST;
+  // One slice: wait for it, let everybody see it, request the slice two ahead into
+  // the stage that was multiplied last time round, multiply.  Every step issues
+  // exactly three loads (past the end it re-requests the last slice into a stage
+  // nobody reads), so "all but the newest three have landed" always means "slice sl
+  // has landed" and the compiler can count the loads in flight at every LDS read.
+  auto step = [&](GemmStage& cur, GemmStage& refill, int sl) __attribute__((always_inline)) {
+    __builtin_amdgcn_s_waitcnt(0x0F73);  // vmcnt(3)
+    // ... and so have everybody else's, and slice sl-1 is consumed.  A bare barrier:
+    // the fences of __syncthreads() would wait for every load in flight, and no wave
+    // stores to LDS with anything but these loads.
+    __builtin_amdgcn_s_barrier();
+    issue(refill, min(sl + 2, slices - 1));
     float2 av[GK2 / 2], bv[GK2 / 2][NQ];
 #pragma unroll
     for (int s2 = 0; s2 < GK2 / 2; ++s2) {
-      av[s2] = As[cur][2 * s2 + h][32 * w + r];
+      av[s2] = cur.A[2 * s2 + h][32 * w + r];
 #pragma unroll
-      for (int q = 0; q < NQ; ++q) bv[s2][q] = Bs[cur][2 * s2 + h][32 * q + r];
+      for (int q = 0; q < NQ; ++q) bv[s2][q] = cur.B[2 * s2 + h][32 * q + r];
     }
 #pragma unroll
     for (int s2 = 0; s2 < GK2 / 2; ++s2) {
@@ -267,7 +274,21 @@ __global__ __launch_bounds__(kT, 2) void binGemmDirect(GemmArgs g) {
         cim[q] = __builtin_amdgcn_mfma_f32_32x32x2f32(nar, b.y, cim[q], 0, 0, 0);
       }
     }
+  };
+
+  issue(stage0, 0);
+  issue(stage1, min(1, slices - 1));
+  int sl = 0;
+  for (; sl + 3 <= slices; sl += 3) {
+    step(stage0, stage2, sl);
+    step(stage1, stage0, sl + 1);
+    step(stage2, stage1, sl + 2);
   }
+  if (sl < slices) {
+    step(stage0, stage2, sl);
+    if (sl + 1 < slices) step(stage1, stage0, sl + 1);
+  }
+  __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): nothing may land in LDS after this wave is gone
 
   float2* Cb = g.C + (long)bin * g.I * g.Jp;
 #pragma unroll

@@ -56,6 +56,26 @@ __device__ __forceinline__ void loadColumnsWindow(const float* src, int sy, int 
   });
 }
 
+// The same two columns for callers whose window geometry differs from lane to
+// lane of a wave (tile descriptors of different planes): the per-row terms are
+// then vector arithmetic, and skipping the loads outside the window (tiles with
+// 9 x 9 filters load 81 of 1024 samples) costs less than clamping every address.
+template <int N>
+__device__ __forceinline__ void loadColumnsWindowPerLane(const float* src, int sy, int sx, int h,
+                                                         int w, int padL, int padU, int l,
+                                                         c32 (&z0)[N / 2], c32 (&z1)[N / 2]) {
+  const int x0 = 2 * l, x1 = 2 * l + 1;
+  auto fetch = [&](int y, int x) {
+    return inWindow(y, x, padU, padL, h, w)
+               ? src[(size_t)(y - padU) * sy + (size_t)(x - padL) * sx] : 0.0f;
+  };
+  staticFor<N / 2>([&](auto jj) {
+    constexpr int j = decltype(jj)::value;
+    z0[j] = c32{fetch(2 * j, x0), fetch(2 * j + 1, x0)};
+    z1[j] = c32{fetch(2 * j, x1), fetch(2 * j + 1, x1)};
+  });
+}
+
 // Column pass (forward): N/2-point FFTs of the two packed columns, real-input
 // fix-up, packed rows written to the plane buffer.
 template <int N>
@@ -120,24 +140,26 @@ template <int N, bool ACC = false>
 __device__ __forceinline__ void storeColumnsWindow(float* dst, int sy, int sx, int h, int w, int padL,
                                                    int padU, int l, const c32 (&z0)[N / 2],
                                                    const c32 (&z1)[N / 2], float scale) {
-  const int x0 = 2 * l, x1 = 2 * l + 1;
-  auto put = [&](int y, int x, float v) {
-    if (inWindow(y, x, padU, padL, h, w)) {
-      float* p = dst + (size_t)(y - padU) * sy + (size_t)(x - padL) * sx;
-      if constexpr (ACC)
-        *p += v * scale;
-      else
-        *p = v * scale;
-    }
+  // The column test is per lane and the same for every row: one masked region per
+  // column.  The row test is wave-uniform: a scalar branch inside it.
+  auto column = [&](int x, const c32 (&z)[N / 2]) __attribute__((always_inline)) {
+    if ((unsigned)(x - padL) >= (unsigned)w) return;
+    float* p = dst + (long)(x - padL) * sx;
+    staticFor<N>([&](auto yy) {
+      constexpr int y = decltype(yy)::value;
+      if ((unsigned)(y - padU) < (unsigned)h) {
+        const c32 v = z[slot<N / 2>(y / 2)];
+        float* q = p + (long)(y - padU) * sy;
+        const float r = (y % 2 ? v.y : v.x) * scale;
+        if constexpr (ACC)
+          *q += r;
+        else
+          *q = r;
+      }
+    });
   };
-  staticFor<N / 2>([&](auto jj) {
-    constexpr int j = decltype(jj)::value;
-    c32 a = z0[slot<N / 2>(j)], c = z1[slot<N / 2>(j)];
-    put(2 * j, x0, a.x);
-    put(2 * j, x1, c.x);
-    put(2 * j + 1, x0, a.y);
-    put(2 * j + 1, x1, c.y);
-  });
+  column(2 * l, z0);
+  column(2 * l + 1, z1);
 }
 
 }  // namespace fbfft_amd

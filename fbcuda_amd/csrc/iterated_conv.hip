@@ -147,7 +147,7 @@ __global__ __launch_bounds__(kThreads) void iteratedConvKernel(ConvArgs a) {
       }
       c32 z0[H], z1[H];
       if (ref.valid) {
-        loadColumnsWindow<N>(ref.p, ref.sy, ref.sx, ref.h, ref.w, ref.padL, ref.padU, l, z0, z1);
+        loadColumnsWindowPerLane<N>(ref.p, ref.sy, ref.sx, ref.h, ref.w, ref.padL, ref.padU, l, z0, z1);
       } else {
 #pragma unroll
         for (int j = 0; j < H; ++j) z0[j] = z1[j] = c32{0.f, 0.f};
