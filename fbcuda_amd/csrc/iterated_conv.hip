@@ -14,13 +14,15 @@
 //   accGradParams    tile, n    ins[t](n, c_a)    outs[t](n, f_w)   a * conj(w) -> weight(f_w, c_a) * scale / N^2
 //
 // The reference gives every (batch, plane) pair its own lanes and recomputes
-// both forward transforms for each of them.  Here a 256-lane workgroup shares
-// BN + FO = 3/4 * (512/N) forward transforms per step among BN * FO products
-// (4 x 8 for N = 32, 8 x 16 for N = 16, 16 x 32 for N = 8): spectra pass through
-// LDS once, and each lane keeps 64 complex accumulators for its own frequency
-// bins in VGPRs across the whole reduction.  Spectral rows 0 and N/2 stay packed
-// as one complex row throughout (fbfft/FFTIteratedConvolution.cuh:161-186), so
-// the inverse needs no re-packing.
+// both forward transforms for each of them.  Here a 512-lane workgroup owns
+// BN x FO products (8 x 8 for N = 32, 16 x 16 for N = 16, 32 x 32 for N = 8) and
+// takes two reduction steps per iteration: its 1024/N plane slots hold the BN + FO
+// forward transforms of both steps, so every lane transforms in every iteration
+// and 2 (BN + FO) transforms feed 2 BN FO products (one transform per 4, 8, 16
+// products).  Spectra pass through LDS once, and each lane keeps 64 complex
+// accumulators for its own frequency bins in VGPRs across the whole reduction.
+// Spectral rows 0 and N/2 travel packed as one complex row through the transforms;
+// the accumulators hold them apart.
 #include "common.h"
 #include "fft2d_core.h"
 #include "fft_regs.h"
@@ -28,7 +30,7 @@
 namespace fbfft_amd {
 namespace {
 
-constexpr int kThreads = 256;
+constexpr int kThreads = 512;
 
 struct ConvArgs {
   const fbfft_tile* ins;
@@ -78,8 +80,10 @@ struct ConvCfg {
   static constexpr int H = N / 2;
   static constexpr int T = N / 2;                  // lanes per plane transform
   static constexpr int SLOTS = kThreads / T;       // concurrent plane transforms
-  static constexpr int FO = SLOTS / 2;             // W planes per workgroup
-  static constexpr int BN = FO / 2;                // A planes per workgroup
+  static constexpr int SPI = 2;                    // reduction steps per iteration
+  static constexpr int FO = SLOTS / (2 * SPI);     // W planes per workgroup
+  static constexpr int BN = FO;                    // A planes per workgroup
+  static constexpr int RA = SLOTS / FO;            // A planes per round of inverse transforms
   static constexpr int RS = PlaneCfg<N>::RS;
   static constexpr int PSZ = H * RS;               // packed plane in LDS (complex)
   static constexpr int PB = H * N;                 // packed bins per plane
@@ -106,7 +110,9 @@ template <int N, int PASS>
 __global__ __launch_bounds__(kThreads) void iteratedConvKernel(ConvArgs a) {
   using C = ConvCfg<N>;
   constexpr int H = C::H, T = C::T, SLOTS = C::SLOTS, FO = C::FO, BN = C::BN, RS = C::RS,
-                PSZ = C::PSZ, PB = C::PB, GRP = C::GRP, NBT = C::NBT, FQ = C::FQ;
+                PSZ = C::PSZ, PB = C::PB, GRP = C::GRP, NBT = C::NBT, FQ = C::FQ, SPI = C::SPI,
+                RA = C::RA;
+  static_assert((BN + FO) * SPI == SLOTS && BN % RA == 0, "slot layout");
   constexpr bool CONJ = (PASS != 1);
   __shared__ __align__(16) c32 lds[SLOTS * PSZ];
 
@@ -130,24 +136,29 @@ __global__ __launch_bounds__(kThreads) void iteratedConvKernel(ConvArgs a) {
       for (int k = 0; k < NBT; ++k) acc[i][j][k] = c32{0.f, 0.f};
 
   c32* plane = lds + s * PSZ;
-  for (int step = 0; step < steps; ++step) {
-    // ---- forward transforms of this step's A and W planes ----
-    if (s < BN + FO) {
+  // slot s transforms plane sj of reduction step SPI * it + su
+  const int su = s / (BN + FO), sj = s % (BN + FO);
+  for (int it = 0; it < (steps + SPI - 1) / SPI; ++it) {
+    // ---- forward transforms of this iteration's A and W planes ----
+    {
+      const int step = SPI * it + su;
       PlaneRef ref;
       if (PASS == 0) {
-        ref = s < BN ? tilePlane(a.ins[tile], a0 + s, step, a.batch)
-                     : weightPlane(a, w0 + s - BN, step);
+        ref = sj < BN ? tilePlane(a.ins[tile], a0 + sj, step, a.batch)
+                      : weightPlane(a, w0 + sj - BN, step);
       } else if (PASS == 1) {
-        ref = s < BN ? tilePlane(a.outs[tile], a0 + s, step, a.batch)
-                     : weightPlane(a, step, w0 + s - BN);
+        ref = sj < BN ? tilePlane(a.outs[tile], a0 + sj, step, a.batch)
+                      : weightPlane(a, step, w0 + sj - BN);
       } else {
-        const int tl = step / a.batch, n = step % a.batch;
-        ref = s < BN ? tilePlane(a.ins[tl], n, a0 + s, a.batch)
-                     : tilePlane(a.outs[tl], n, w0 + s - BN, a.batch);
+        // past the last step the tile index is clamped; the plane is zeroed below
+        const int tl = min(step / a.batch, a.numTiles - 1), n = step % a.batch;
+        ref = sj < BN ? tilePlane(a.ins[tl], n, a0 + sj, a.batch)
+                      : tilePlane(a.outs[tl], n, w0 + sj - BN, a.batch);
       }
       c32 z0[H], z1[H];
-      if (ref.valid) {
-        loadColumnsWindowPerLane<N>(ref.p, ref.sy, ref.sx, ref.h, ref.w, ref.padL, ref.padU, l, z0, z1);
+      if (ref.valid && step < steps) {
+        loadColumnsWindowPerLane<N>(ref.p, ref.sy, ref.sx, ref.h, ref.w, ref.padL, ref.padU, l, z0,
+                                    z1);
       } else {
 #pragma unroll
         for (int j = 0; j < H; ++j) z0[j] = z1[j] = c32{0.f, 0.f};
@@ -155,61 +166,75 @@ __global__ __launch_bounds__(kThreads) void iteratedConvKernel(ConvArgs a) {
       columnPassForward<N>(z0, z1, plane, l);
     }
     __syncthreads();
-    if (s < BN + FO) rowPassInPlace<N, true>(plane, l);
+    rowPassInPlace<N, true>(plane, l);
     __syncthreads();
 
     // ---- acc[a][w] += A_a (x) W_w on this lane's bins ----
+    // Packed row 0 holds P[x] = F0[x] + i*FH[x], the Hermitian spectra of the two
+    // real rows 0 and N/2.  Its lanes do not multiply packed values (that takes both
+    // products in every lane, fbfft/FFTIteratedConvolution.cuh:161-186): lane x < N/2
+    // accumulates the row-0 product at x and lane N/2 + x the row-N/2 product at x,
+    // one complex product each like every other bin.  x = 0 carries the real values
+    // at 0 and N/2 of its row as (re, im) and multiplies them separately.
+#pragma unroll 1
+    for (int u = 0; u < SPI; ++u) {
+      const c32* ldsu = lds + u * (BN + FO) * PSZ;
 #pragma unroll
-    for (int nb = 0; nb < NBT; ++nb) {
-      const int bin = bin0 + kThreads * nb;
-      const int r = bin / N, x = bin % N;
-      const int o = r * RS + x;
-      if (r != 0) {
+      for (int nb = 0; nb < NBT; ++nb) {
+        const int bin = bin0 + kThreads * nb;
+        const int r = bin / N, x = bin % N;
         c32 wv[FQ];
+        if (r != 0) {
+          const int o = r * RS + x;
 #pragma unroll
-        for (int q = 0; q < FQ; ++q) wv[q] = lds[(BN + gidx + GRP * q) * PSZ + o];
+          for (int q = 0; q < FQ; ++q) wv[q] = ldsu[(BN + gidx + GRP * q) * PSZ + o];
 #pragma unroll
-        for (int i = 0; i < BN; ++i) {
-          const c32 av = lds[i * PSZ + o];
+          for (int i = 0; i < BN; ++i) {
+            const c32 av = ldsu[i * PSZ + o];
 #pragma unroll
-          for (int q = 0; q < FQ; ++q) {
-            c32 p = prod<CONJ>(av, wv[q]);
-            acc[i][q][nb].x += p.x;
-            acc[i][q][nb].y += p.y;
+            for (int q = 0; q < FQ; ++q) {
+              const c32 p = prod<CONJ>(av, wv[q]);
+              acc[i][q][nb].x += p.x;
+              acc[i][q][nb].y += p.y;
+            }
           }
-        }
-      } else if (x != 0) {
-        // packed row: two real-row spectra per value, multiplied separately and re-packed
-        const int om = (N - x);
-        c32 w0v[FQ], wHv[FQ];
+        } else {
+          const int xx = x & (H - 1);
+          const bool second = x >= H;
+          if (xx != 0) {
+            auto half = [&](const c32* p) __attribute__((always_inline)) {
+              c32 r0, rH;
+              unpack0(p[xx], p[N - xx], &r0, &rH);
+              return second ? rH : r0;
+            };
 #pragma unroll
-        for (int q = 0; q < FQ; ++q) {
-          const c32* wp = lds + (BN + gidx + GRP * q) * PSZ;
-          unpack0(wp[x], wp[om], &w0v[q], &wHv[q]);
-        }
+            for (int q = 0; q < FQ; ++q) wv[q] = half(ldsu + (BN + gidx + GRP * q) * PSZ);
 #pragma unroll
-        for (int i = 0; i < BN; ++i) {
-          const c32* ap = lds + i * PSZ;
-          c32 a0v, aHv;
-          unpack0(ap[x], ap[om], &a0v, &aHv);
+            for (int i = 0; i < BN; ++i) {
+              const c32 av = half(ldsu + i * PSZ);
 #pragma unroll
-          for (int q = 0; q < FQ; ++q) {
-            c32 p0 = prod<CONJ>(a0v, w0v[q]);
-            c32 pH = prod<CONJ>(aHv, wHv[q]);
-            acc[i][q][nb].x += p0.x - pH.y;  // p0 + i * pH
-            acc[i][q][nb].y += p0.y + pH.x;
-          }
-        }
-      } else {
-        // x = 0: both halves are real (fbfft/FFTIteratedConvolution.cuh:176-180)
+              for (int q = 0; q < FQ; ++q) {
+                const c32 p = prod<CONJ>(av, wv[q]);
+                acc[i][q][nb].x += p.x;
+                acc[i][q][nb].y += p.y;
+              }
+            }
+          } else {
+            auto ends = [&](const c32* p) __attribute__((always_inline)) {
+              const c32 p0 = p[0], pH = p[H];
+              return second ? c32{p0.y, pH.y} : c32{p0.x, pH.x};
+            };
 #pragma unroll
-        for (int i = 0; i < BN; ++i) {
-          const c32 av = lds[i * PSZ];
+            for (int q = 0; q < FQ; ++q) wv[q] = ends(ldsu + (BN + gidx + GRP * q) * PSZ);
 #pragma unroll
-          for (int q = 0; q < FQ; ++q) {
-            const c32 wv = lds[(BN + gidx + GRP * q) * PSZ];
-            acc[i][q][nb].x += av.x * wv.x;
-            acc[i][q][nb].y += av.y * wv.y;
+            for (int i = 0; i < BN; ++i) {
+              const c32 av = ends(ldsu + i * PSZ);
+#pragma unroll
+              for (int q = 0; q < FQ; ++q) {
+                acc[i][q][nb].x += av.x * wv[q].x;
+                acc[i][q][nb].y += av.y * wv[q].y;
+              }
+            }
           }
         }
       }
@@ -217,26 +242,60 @@ __global__ __launch_bounds__(kThreads) void iteratedConvKernel(ConvArgs a) {
     __syncthreads();
   }
 
-  // ---- inverse transforms, 2 A planes x FO W planes per round ----
+  // ---- inverse transforms, RA A planes x FO W planes per round ----
   const float norm = (PASS == 2 ? a.scale : 1.0f) / (float)(N * N);
 #pragma unroll
-  for (int rd = 0; rd < BN / 2; ++rd) {
+  for (int rd = 0; rd < BN / RA; ++rd) {
+    // Row-0 lanes park their value in the plane's padding (columns N, N+1 of row
+    // x/2: N spare cells per plane) where the partner lane finds it.
 #pragma unroll
-    for (int ii = 0; ii < 2; ++ii)
+    for (int ii = 0; ii < RA; ++ii)
 #pragma unroll
       for (int q = 0; q < FQ; ++q)
 #pragma unroll
         for (int nb = 0; nb < NBT; ++nb) {
           const int bin = bin0 + kThreads * nb;
-          lds[(ii * FO + gidx + GRP * q) * PSZ + (bin / N) * RS + bin % N] = acc[2 * rd + ii][q][nb];
+          const int x = bin % N;
+          const int o = bin < N ? (x / 2) * RS + N + x % 2 : (bin / N) * RS + x;
+          lds[(ii * FO + gidx + GRP * q) * PSZ + o] = acc[RA * rd + ii][q][nb];
         }
+    __syncthreads();
+    // Row 0 back to its packed form Q[x] = S0[x] + i*SH[x], Q[N-x] = conj(S0[x]) +
+    // i*conj(SH[x]): the lane holding S0[x] fetches SH[x] and writes Q[x], the lane
+    // holding SH[x] fetches S0[x] and writes Q[N-x]; the two real pairs swap halves.
+#pragma unroll
+    for (int nb = 0; nb < NBT; ++nb) {
+      const int bin = bin0 + kThreads * nb;
+      if (bin < N) {
+        const int x = bin, xx = x & (H - 1);
+        const bool second = x >= H;
+        const int px = second ? xx : H + xx;  // partner's x
+        const int src = (px / 2) * RS + N + px % 2;
+        const int dst = xx == 0 ? x : second ? N - xx : x;
+#pragma unroll
+        for (int ii = 0; ii < RA; ++ii)
+#pragma unroll
+          for (int q = 0; q < FQ; ++q) {
+            c32* pl = lds + (ii * FO + gidx + GRP * q) * PSZ;
+            const c32 mine = acc[RA * rd + ii][q][nb];
+            const c32 other = pl[src];
+            c32 v;
+            if (xx == 0)
+              v = second ? c32{other.y, mine.y} : c32{mine.x, other.x};
+            else
+              v = second ? c32{other.x + mine.y, mine.x - other.y}
+                         : c32{mine.x - other.y, mine.y + other.x};
+            pl[dst] = v;
+          }
+      }
+    }
     __syncthreads();
     rowPassInPlace<N, false>(plane, l);
     __syncthreads();
     {
       c32 z0[H], z1[H];
       columnPassInverse<N>(plane, l, z0, z1);
-      const int ai = a0 + 2 * rd + s / FO;
+      const int ai = a0 + RA * rd + s / FO;
       const int wi = w0 + s % FO;
       PlaneRef ref;
       if (PASS == 0)
