@@ -253,42 +253,126 @@ __global__ __launch_bounds__(LargeCfg<N>::THREADS) void fft2dLargeInverse(CplxVi
   });
   __syncthreads();
 
-  // ---- row pass (inverse): lane y.  (Splitting this pass over two lanes as the
-  // forward kernel does for N = 128 needs the fix-up as a separate LDS pass and
-  // measured slower: 149 us against 126 us for 4096 planes.) ----
-  c32 z[H];
-  if (t < N) {
-    const c32* row = cb + t * YS;
-    realFixupInverseFetch<H>([&](auto kk) { return row[decltype(kk)::value]; }, z);
-    difFFT<H, false>(z);
-  }
-  __syncthreads();
-  if (t < N) {
-    float* row = buf + t * RSF;
-    staticFor<H / 2>([&](auto mm) {
-      constexpr int m = decltype(mm)::value;
-      c32 a = z[slot<H>(2 * m)], c = z[slot<H>(2 * m + 1)];
-      *reinterpret_cast<float4*>(row + 4 * m) = float4{a.x, a.y, c.x, c.y};
-    });
-  }
-  __syncthreads();
+  if constexpr (THREADS == N) {
+    // ---- row pass (inverse): lane y ----
+    c32 z[H];
+    {
+      const c32* row = cb + t * YS;
+      realFixupInverseFetch<H>([&](auto kk) { return row[decltype(kk)::value]; }, z);
+      difFFT<H, false>(z);
+    }
+    __syncthreads();
+    {
+      float* row = buf + t * RSF;
+      staticFor<H / 2>([&](auto mm) {
+        constexpr int m = decltype(mm)::value;
+        c32 a = z[slot<H>(2 * m)], c = z[slot<H>(2 * m + 1)];
+        *reinterpret_cast<float4*>(row + 4 * m) = float4{a.x, a.y, c.x, c.y};
+      });
+    }
+    __syncthreads();
 
-  // ---- copy out, cropped to the window real covers ----
-  if constexpr (FAST_REAL) {
-    float4* dst = reinterpret_cast<float4*>(real.data + (size_t)b * real.sb);
-    const int rs4 = real.sy / 4;
-    staticFor<C::F4_REAL / THREADS>([&](auto ii) {
-      constexpr int i = decltype(ii)::value;
-      const int q = t + THREADS * i;
-      const int y = q / (N / 4), x4 = q % (N / 4);
-      dst[(size_t)y * rs4 + x4] = *reinterpret_cast<const float4*>(buf + y * RSF + 4 * x4);
-    });
+    // ---- copy out, cropped to the window real covers ----
+    if constexpr (FAST_REAL) {
+      float4* dst = reinterpret_cast<float4*>(real.data + (size_t)b * real.sb);
+      const int rs4 = real.sy / 4;
+      staticFor<C::F4_REAL / THREADS>([&](auto ii) {
+        constexpr int i = decltype(ii)::value;
+        const int q = t + THREADS * i;
+        const int y = q / (N / 4), x4 = q % (N / 4);
+        dst[(size_t)y * rs4 + x4] = *reinterpret_cast<const float4*>(buf + y * RSF + 4 * x4);
+      });
+    } else {
+      float* dst = real.data + (size_t)b * real.sb;
+      for (int q = t; q < N * N; q += THREADS) {
+        const int y = q / N, x = q % N;
+        if (inWindow(y, x, padU, padL, real.h, real.w))
+          dst[(size_t)(y - padU) * real.sy + (size_t)(x - padL) * real.sx] = buf[y * RSF + x];
+      }
+    }
   } else {
-    float* dst = real.data + (size_t)b * real.sb;
-    for (int q = t; q < N * N; q += THREADS) {
-      const int y = q / N, x = q % N;
-      if (inWindow(y, x, padU, padL, real.h, real.w))
-        dst[(size_t)(y - padU) * real.sy + (size_t)(x - padL) * real.sx] = buf[y * RSF + x];
+    // ---- row pass (inverse) over two lanes per row y.  The H-point inverse
+    // transform of z splits by the parity of its input index: lane g takes
+    // z[2m + g], whose real-input fix-up pairs (k, H - k) have the same parity, so
+    // neither lane repeats the other's fix-up.  With E = IFFT(z even), O = IFFT(z odd)
+    // the result is x[j] = E[j] + w^j O[j], x[j + H/2] = E[j] - w^j O[j], w = e^{2 pi i/H}.
+    // Lane 1 scales its half by w^j; the sum and difference are formed on the way
+    // out of LDS.  g is the same for a whole wave. ----
+    static_assert(THREADS == 2 * N, "two lanes per row");
+    constexpr int Q = H / 2;  // points per lane
+    const int y = t % N, g = t / N;
+    c32 zz[Q];
+    {
+      const c32* row = cb + y * YS;
+      auto pairFix = [&](auto kk, c32& zk, c32& zhk) __attribute__((always_inline)) {
+        constexpr int k = decltype(kk)::value;
+        const c32 a = row[k], bb = row[H - k];
+        const c32 e = c32{a.x + bb.x, a.y - bb.y};
+        const c32 d = c32{a.x - bb.x, a.y + bb.y};
+        const c32 o = mulRoot<N, k, false>(d);
+        zk = c32{e.x - o.y, e.y + o.x};
+        zhk = c32{e.x + o.y, o.x - e.y};
+      };
+      if (g == 0) {
+        const c32 p0 = row[0];
+        zz[0] = c32{p0.x + p0.y, p0.x - p0.y};
+        staticFor<Q / 2 - 1>([&](auto mm) {
+          constexpr int k = 2 * (decltype(mm)::value + 1);  // 2, 4, ..., H/2 - 2
+          pairFix(std::integral_constant<int, k>{}, zz[k / 2], zz[(H - k) / 2]);
+        });
+        const c32 a = row[H / 2];
+        zz[Q / 2] = c32{2.0f * a.x, -2.0f * a.y};
+      } else {
+        staticFor<Q / 2>([&](auto mm) {
+          constexpr int k = 2 * decltype(mm)::value + 1;    // 1, 3, ..., H/2 - 1
+          pairFix(std::integral_constant<int, k>{}, zz[(k - 1) / 2], zz[(H - k - 1) / 2]);
+        });
+      }
+    }
+    difFFT<Q, false>(zz);
+    if (g == 1) {
+      staticFor<Q>([&](auto jj) {
+        constexpr int j = decltype(jj)::value;
+        zz[slot<Q>(j)] = mulRoot<H, j, false>(zz[slot<Q>(j)]);
+      });
+    }
+    __syncthreads();
+    {
+      // row y of the staging buffer: E as floats [0, H), w^j O as floats [H, N)
+      float* row = buf + y * RSF + H * g;
+      staticFor<Q / 2>([&](auto mm) {
+        constexpr int m = decltype(mm)::value;
+        c32 a = zz[slot<Q>(2 * m)], c = zz[slot<Q>(2 * m + 1)];
+        *reinterpret_cast<float4*>(row + 4 * m) = float4{a.x, a.y, c.x, c.y};
+      });
+    }
+    __syncthreads();
+
+    // ---- copy out, cropped to the window real covers: real samples 2j, 2j+1 are
+    // (re, im) of x[j] ----
+    if constexpr (FAST_REAL) {
+      float4* dst = reinterpret_cast<float4*>(real.data + (size_t)b * real.sb);
+      const int rs4 = real.sy / 4;
+      staticFor<C::F4_REAL / THREADS>([&](auto ii) {
+        constexpr int i = decltype(ii)::value;
+        const int q = t + THREADS * i;
+        const int yy = q / (N / 4), x4 = q % (N / 4);
+        const int f = (4 * x4) % H;  // float offset of E[j], j = 2*x4 mod H/2
+        const float4 e = *reinterpret_cast<const float4*>(buf + yy * RSF + f);
+        const float4 w = *reinterpret_cast<const float4*>(buf + yy * RSF + H + f);
+        const float sg = 4 * x4 < H ? 1.0f : -1.0f;
+        dst[(size_t)yy * rs4 + x4] =
+            float4{e.x + sg * w.x, e.y + sg * w.y, e.z + sg * w.z, e.w + sg * w.w};
+      });
+    } else {
+      float* dst = real.data + (size_t)b * real.sb;
+      for (int q = t; q < N * N; q += THREADS) {
+        const int yy = q / N, x = q % N;
+        if (inWindow(yy, x, padU, padL, real.h, real.w)) {
+          const float e = buf[yy * RSF + x % H], w = buf[yy * RSF + H + x % H];
+          dst[(size_t)(yy - padU) * real.sy + (size_t)(x - padL) * real.sx] = x < H ? e + w : e - w;
+        }
+      }
     }
   }
 }
