@@ -195,17 +195,25 @@ __device__ __forceinline__ void loadToLds(const float2* src, float2* ldsWaveBase
                                    (__attribute__((address_space(3))) void*)ldsWaveBase, 16, 0, 0);
 }
 
+template <int TI>
 struct GemmStage {
-  float2 A[GK2][GI];
+  float2 A[GK2][TI];
   float2 B[GK2][GJ2];
 };
 
+// TI = 128: wave w owns rows 32w.. and both 32-column halves of the 64 columns.
+// TI = 64 (few rows, or too few 128-row tiles to balance the chip): wave w owns rows
+// 32 (w % 2).. and columns 32 (w / 2)..
+template <int TI>
 __global__ __launch_bounds__(kT, 4) void binGemmDirect(GemmArgs g) {
-  constexpr int NQ = GJ2 / 32;
+  static_assert(TI == 128 || TI == 64, "tile rows");
+  constexpr int NQ = TI == 128 ? 2 : 1;
+  constexpr int LOADS = TI == 128 ? 3 : 2;  // global->LDS instructions per wave and slice
+  using Stage = GemmStage<TI>;
   // three separate variables, not one array: the compiler tracks pending
   // global->LDS loads per LDS variable, so reading one stage does not wait for the
   // loads still in flight into the other two
-  __shared__ __align__(16) GemmStage stage0, stage1, stage2;
+  __shared__ __align__(16) Stage stage0, stage1, stage2;
   const int t = threadIdx.x;
   const int lane = t % 64, w = t / 64;
   const int r = lane % 32, h = lane / 32;
@@ -216,12 +224,14 @@ __global__ __launch_bounds__(kT, 4) void binGemmDirect(GemmArgs g) {
   if (logical >= total) return;
   const int bin = logical / (g.IT * g.JT);
   const int rem = logical % (g.IT * g.JT);
-  const int i0 = (rem / g.JT) * GI, j0 = (rem % g.JT) * GJ2;
+  const int i0 = (rem / g.JT) * TI, j0 = (rem % g.JT) * GJ2;
+  const int rb = TI == 128 ? w : w % 2;  // 32-row block of this wave
+  const int cb = TI == 128 ? 0 : w / 2;  // first 32-column block of this wave
 
   const float2* Ab = g.A + (long)bin * g.Kp * g.Ip;
   const float2* Bb = g.B + (long)bin * g.Kp * g.Jp;
   // per-lane source columns, clamped into the padded arrays
-  const int ia = min(i0 + 2 * lane, g.Ip - 2);
+  const int ia = min(i0 + 2 * (TI == 128 ? lane : lane % 32), g.Ip - 2);
   const int jb = min(j0 + 2 * (lane % 32), g.Jp - 2);
 
   floatx16 cre[NQ], cim[NQ];
@@ -234,21 +244,25 @@ __global__ __launch_bounds__(kT, 4) void binGemmDirect(GemmArgs g) {
     }
 
   const int slices = g.Kp / GK2;
-  // wave w moves rows 2w, 2w+1 of A and rows 2w, 2w+1 of B of a slice: 3 instructions
-  auto issue = [&](GemmStage& st, int sl) __attribute__((always_inline)) {
+  // wave w moves rows 2w, 2w+1 of A and rows 2w, 2w+1 of B of a slice: LOADS instructions
+  auto issue = [&](Stage& st, int sl) __attribute__((always_inline)) {
     const int k0 = sl * GK2;
-    loadToLds(Ab + (long)(k0 + 2 * w) * g.Ip + ia, &st.A[2 * w][0]);
-    loadToLds(Ab + (long)(k0 + 2 * w + 1) * g.Ip + ia, &st.A[2 * w + 1][0]);
+    if constexpr (TI == 128) {
+      loadToLds(Ab + (long)(k0 + 2 * w) * g.Ip + ia, &st.A[2 * w][0]);
+      loadToLds(Ab + (long)(k0 + 2 * w + 1) * g.Ip + ia, &st.A[2 * w + 1][0]);
+    } else {
+      loadToLds(Ab + (long)(k0 + 2 * w + h) * g.Ip + ia, &st.A[2 * w][0]);
+    }
     loadToLds(Bb + (long)(k0 + 2 * w + h) * g.Jp + jb, &st.B[2 * w][0]);
   };
 
   // One slice: wait for it, let everybody see it, request the slice two ahead into
   // the stage that was multiplied last time round, multiply.  Every step issues
-  // exactly three loads (past the end it re-requests the last slice into a stage
-  // nobody reads), so "all but the newest three have landed" always means "slice sl
+  // exactly LOADS loads (past the end it re-requests the last slice into a stage
+  // nobody reads), so "all but the newest LOADS have landed" always means "slice sl
   // has landed" and the compiler can count the loads in flight at every LDS read.
-  auto step = [&](GemmStage& cur, GemmStage& refill, int sl) __attribute__((always_inline)) {
-    __builtin_amdgcn_s_waitcnt(0x0F73);  // vmcnt(3)
+  auto step = [&](Stage& cur, Stage& refill, int sl) __attribute__((always_inline)) {
+    __builtin_amdgcn_s_waitcnt(0x0F70 | LOADS);  // vmcnt(LOADS)
     // ... and so have everybody else's, and slice sl-1 is consumed.  A bare barrier:
     // the fences of __syncthreads() would wait for every load in flight, and no wave
     // stores to LDS with anything but these loads.
@@ -257,9 +271,9 @@ __global__ __launch_bounds__(kT, 4) void binGemmDirect(GemmArgs g) {
     float2 av[GK2 / 2], bv[GK2 / 2][NQ];
 #pragma unroll
     for (int s2 = 0; s2 < GK2 / 2; ++s2) {
-      av[s2] = cur.A[2 * s2 + h][32 * w + r];
+      av[s2] = cur.A[2 * s2 + h][32 * rb + r];
 #pragma unroll
-      for (int q = 0; q < NQ; ++q) bv[s2][q] = cur.B[2 * s2 + h][32 * q + r];
+      for (int q = 0; q < NQ; ++q) bv[s2][q] = cur.B[2 * s2 + h][32 * (cb + q) + r];
     }
 #pragma unroll
     for (int s2 = 0; s2 < GK2 / 2; ++s2) {
@@ -293,11 +307,11 @@ __global__ __launch_bounds__(kT, 4) void binGemmDirect(GemmArgs g) {
   float2* Cb = g.C + (long)bin * g.I * g.Jp;
 #pragma unroll
   for (int q = 0; q < NQ; ++q) {
-    const int j = j0 + 32 * q + r;
+    const int j = j0 + 32 * (cb + q) + r;
     if (j >= g.Jp) continue;
 #pragma unroll
     for (int v = 0; v < 16; ++v) {
-      const int i = i0 + 32 * w + 8 * (v / 4) + 4 * h + v % 4;
+      const int i = i0 + 32 * rb + 8 * (v / 4) + 4 * h + v % 4;
       if (i < g.I) Cb[(long)i * g.Jp + j] = float2{cre[q][v] * g.invNorm, cim[q][v] * g.invNorm};
     }
   }
@@ -353,10 +367,19 @@ int runPipeline(PlaneSet x, PlaneSet y, PlaneSet out, bool conjY, float scale, b
   g.Ip = Ip;
   g.Jp = Jp;
   g.Kp = Kp;
-  g.IT = ceilDiv(I, GI);
   g.JT = ceilDiv(Jp, GJ2);
   g.invNorm = 1.0f / (float)(N * N);
-  binGemmDirect<<<dim3(roundUp(bins * g.IT * g.JT, 8)), dim3(kT), 0, s>>>(g);
+  // 64-row tiles when they waste fewer rows, or when 128-row tiles would leave the
+  // chip with fewer than eight workgroups per CU to balance (measured equal or
+  // faster there: 84 -> 62 us for 64 x 192 x 128 per bin, 77 -> 69 us for 128 x 64 x 192)
+  const bool small = roundUp(I, 64) < roundUp(I, GI) || (long)bins * ceilDiv(I, GI) * g.JT < 8 * 256;
+  if (small) {
+    g.IT = ceilDiv(I, 64);
+    binGemmDirect<64><<<dim3(roundUp(bins * g.IT * g.JT, 8)), dim3(kT), 0, s>>>(g);
+  } else {
+    g.IT = ceilDiv(I, GI);
+    binGemmDirect<GI><<<dim3(roundUp(bins * g.IT * g.JT, 8)), dim3(kT), 0, s>>>(g);
+  }
   if (accumulate)
     inverseBinMajor<N, true><<<dim3(Jp / SL, I), dim3(kT), 0, s>>>(SC, I, Jp, out, scale);
   else
