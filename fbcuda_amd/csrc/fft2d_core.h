@@ -140,26 +140,28 @@ template <int N, bool ACC = false>
 __device__ __forceinline__ void storeColumnsWindow(float* dst, int sy, int sx, int h, int w, int padL,
                                                    int padU, int l, const c32 (&z0)[N / 2],
                                                    const c32 (&z1)[N / 2], float scale) {
-  // The column test is per lane and the same for every row: one masked region per
-  // column.  The row test is wave-uniform: a scalar branch inside it.
-  auto column = [&](int x, const c32 (&z)[N / 2]) __attribute__((always_inline)) {
-    if ((unsigned)(x - padL) >= (unsigned)w) return;
-    float* p = dst + (long)(x - padL) * sx;
-    staticFor<N>([&](auto yy) {
-      constexpr int y = decltype(yy)::value;
-      if ((unsigned)(y - padU) < (unsigned)h) {
-        const c32 v = z[slot<N / 2>(y / 2)];
-        float* q = p + (long)(y - padU) * sy;
-        const float r = (y % 2 ? v.y : v.x) * scale;
-        if constexpr (ACC)
-          *q += r;
-        else
-          *q = r;
-      }
-    });
+  // The column tests are per lane and the same for every row; the row test is
+  // wave-uniform (a scalar branch).  The two columns of a row are stored back to
+  // back so that both halves of a cache line reach L2 together.
+  const int xa = 2 * l - padL, xb = xa + 1;
+  const bool va = (unsigned)xa < (unsigned)w, vb = (unsigned)xb < (unsigned)w;
+  float* pa = dst + (long)xa * sx;
+  float* pb = dst + (long)xb * sx;
+  auto put = [&](float* q, float r) __attribute__((always_inline)) {
+    if constexpr (ACC)
+      *q += r * scale;
+    else
+      *q = r * scale;
   };
-  column(2 * l, z0);
-  column(2 * l + 1, z1);
+  staticFor<N>([&](auto yy) {
+    constexpr int y = decltype(yy)::value;
+    if ((unsigned)(y - padU) < (unsigned)h) {
+      const long oy = (long)(y - padU) * sy;
+      const c32 a = z0[slot<N / 2>(y / 2)], c = z1[slot<N / 2>(y / 2)];
+      if (va) put(pa + oy, y % 2 ? a.y : a.x);
+      if (vb) put(pb + oy, y % 2 ? c.y : c.x);
+    }
+  });
 }
 
 }  // namespace fbfft_amd
