@@ -89,9 +89,17 @@ def cpu_baseline(x_host, N, budget_s=12.0):
         O.fbfft2d(x_host, N)
     dt = (time.perf_counter() - t0) / reps
     gbs = x_host.shape[0] * plane_bytes(N) / dt / 1e9
+    # one thread, a few passes, for scale
+    O.set_num_threads(1)
+    t0 = time.perf_counter()
+    for _ in range(3):
+        O.fbfft2d(x_host, N)
+    dt1 = (time.perf_counter() - t0) / 3
+    O.set_num_threads(threads)
     return {"value": round(gbs, 3), "unit": "GB/s", "cores": threads, "kind": "port",
             "sample": "%d passes of the full %d-plane %dx%d R2C batch, OpenMP over planes, "
-                      "%.3f s per pass" % (reps, x_host.shape[0], N, N, dt)}
+                      "%.3f s per pass" % (reps, x_host.shape[0], N, N, dt),
+            "single_thread_GBps": round(x_host.shape[0] * plane_bytes(N) / dt1 / 1e9, 3)}
 
 
 def measured_traffic():
@@ -300,6 +308,17 @@ def main():
             extra["r2c_%dx%d_b%d_GBps" % (n2, n2, b2)] = round(nb / lf / 1e9, 1)
             extra["c2r_%dx%d_b%d_GBps" % (n2, n2, b2)] = round(nb / li / 1e9, 1)
             del x2, s2
+        # configs[0] (1D, 32 points, 4096 rows: launch-bound) and the largest 1D size
+        for n1, b1 in ((32, 4096), (256, 1 << 18)):
+            x1 = synth.uniform((b1, n1), seed=0, device=dev)
+            s1 = torch.empty((b1, n1 // 2 + 1, 2), device=dev)
+            _, lf = timed(prepared("fbfft_r2c_1d", F, x1, s1, 0), 50, 5, torch)
+            _, li = timed(prepared("fbfft_c2r_1d", F, x1, s1, 0), 50, 5, torch)
+            nb = b1 * (4 * n1 + 8 * (n1 // 2 + 1))
+            extra["r2c_1d_%d_b%d_us" % (n1, b1)] = round(lf * 1e6, 2)
+            extra["c2r_1d_%d_b%d_us" % (n1, b1)] = round(li * 1e6, 2)
+            extra["r2c_1d_%d_b%d_GBps" % (n1, b1)] = round(nb / lf / 1e9, 1)
+            del x1, s1
         conv_extras(F, synth, torch, dev, extra)
 
     out = {
