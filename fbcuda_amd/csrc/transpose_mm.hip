@@ -15,7 +15,8 @@
 //
 // Per 4-deep slice of k the workgroup stages opA and opB in LDS split into real
 // and imaginary planes [bin][k][row] (conjugation folded into the sign of the
-// imaginary plane) while the next slice is already in flight in registers; each
+// imaginary plane), two buffers deep, while the slice after next is in flight in
+// registers; each
 // wave then issues v_mfma_f32_32x32x2_f32, four real products per complex
 // product: Cre += Ar*Br + (-Ai)*Bi, Cim += Ar*Bi + Ai*Br.  C leaves through LDS
 // so that stores cover whole runs.  Only this contraction uses MFMA; it is the
@@ -33,7 +34,8 @@ constexpr int XS = KC * 64 + 4;   // bin stride of an LDS plane (dwords): the 4 
 constexpr int PLANE = XB * XS;    // one of Ar, Ai, Br, Bi
 constexpr int CSTR = XB + 1;      // padded bin stride of the C staging buffer (complex)
 constexpr int STAGE_FLOATS = 8 * TJ * CSTR * 2;
-constexpr int LDS_FLOATS = (4 * PLANE > STAGE_FLOATS) ? 4 * PLANE : STAGE_FLOATS;
+constexpr int BUF = 4 * PLANE;    // Ar, Ai, Br, Bi of one slice
+constexpr int LDS_FLOATS = (2 * BUF > STAGE_FLOATS) ? 2 * BUF : STAGE_FLOATS;
 
 struct MMArgs {
   const float* A;
@@ -57,6 +59,10 @@ struct Fetch {
   float4 v[KC / 2];
 };
 
+// Every load is issued unconditionally at an address clamped into the operand; the
+// values outside it are zeroed only when the slice is parked in LDS one iteration
+// later, so nothing waits for a load between its issue and the products of the
+// current slice.  VEC4 additionally needs XY even (a bin pair never straddles the end).
 template <bool VEC4>
 __device__ __forceinline__ Fetch fetchSlice(const float* base, long rowStride, long kStride,
                                             int rows, int row0, int K, int k0, int XY, int x0,
@@ -66,50 +72,47 @@ __device__ __forceinline__ Fetch fetchSlice(const float* base, long rowStride, l
   const int x = x0 + 2 * p;
   const int e = t / 4;
   const int row = row0 + e % 64;
+  const float* src0 = base + (long)min(row, rows - 1) * rowStride + 2L * min(x, XY - (VEC4 ? 2 : 1));
+  const long x1off = x + 1 < XY ? 2 : 0;
 #pragma unroll
   for (int u = 0; u < KC / 2; ++u) {
     const int k = k0 + e / 64 + 2 * u;
-    f.v[u] = float4{0.f, 0.f, 0.f, 0.f};
-    if (row < rows && k < K && x < XY) {
-      const float* src = base + (long)row * rowStride + (long)k * kStride + 2L * x;
-      if (VEC4 && x + 1 < XY) {
-        f.v[u] = *reinterpret_cast<const float4*>(src);
-      } else {
-        float2 a = *reinterpret_cast<const float2*>(src);
-        f.v[u].x = a.x;
-        f.v[u].y = a.y;
-        if (x + 1 < XY) {
-          float2 b = *reinterpret_cast<const float2*>(src + 2);
-          f.v[u].z = b.x;
-          f.v[u].w = b.y;
-        }
-      }
+    const float* src = src0 + (long)min(k, K - 1) * kStride;
+    if constexpr (VEC4) {
+      f.v[u] = *reinterpret_cast<const float4*>(src);
+    } else {
+      const float2 a = *reinterpret_cast<const float2*>(src);
+      const float2 b = *reinterpret_cast<const float2*>(src + x1off);
+      f.v[u] = float4{a.x, a.y, b.x, b.y};
     }
   }
   return f;
 }
 
-__device__ __forceinline__ void stashSlice(float* re, float* im, const Fetch& f, float sign, int t) {
+// Parks a fetched slice (k0 .. k0 + KC) in its LDS planes, zeroing what lies outside
+// the operand.
+__device__ __forceinline__ void stashSlice(float* re, float* im, const Fetch& f, float sign,
+                                           int rows, int row0, int K, int k0, int XY, int x0,
+                                           int t) {
   const int p = t % 4;
   const int e = t / 4;
+  const int x = x0 + 2 * p;
+  const bool ok0 = row0 + e % 64 < rows && x < XY;
+  const bool okX1 = x + 1 < XY;
 #pragma unroll
   for (int u = 0; u < KC / 2; ++u) {
     const int o = (e / 64 + 2 * u) * 64 + e % 64;
-    re[(2 * p) * XS + o] = f.v[u].x;
-    im[(2 * p) * XS + o] = sign * f.v[u].y;
-    re[(2 * p + 1) * XS + o] = f.v[u].z;
-    im[(2 * p + 1) * XS + o] = sign * f.v[u].w;
+    const bool ok = ok0 && k0 + e / 64 + 2 * u < K;
+    re[(2 * p) * XS + o] = ok ? f.v[u].x : 0.f;
+    im[(2 * p) * XS + o] = ok ? sign * f.v[u].y : 0.f;
+    re[(2 * p + 1) * XS + o] = ok && okX1 ? f.v[u].z : 0.f;
+    im[(2 * p + 1) * XS + o] = ok && okX1 ? sign * f.v[u].w : 0.f;
   }
 }
 
 template <bool VEC4>
 __global__ __launch_bounds__(THREADS) void transposeMMKernel(MMArgs a) {
-  __shared__ __align__(8) float lds[LDS_FLOATS];
-  float* Ar = lds;
-  float* Ai = lds + PLANE;
-  float* Br = lds + 2 * PLANE;
-  float* Bi = lds + 3 * PLANE;
-
+  __shared__ __align__(8) float lds[LDS_FLOATS];  // two slice buffers; later the C staging area
   const int t = threadIdx.x;
   const int lane = t % 64, w = t / 64;
   // Workgroups are dealt round-robin to the 8 XCDs, each with its own L2.  Give
@@ -139,18 +142,35 @@ __global__ __launch_bounds__(THREADS) void transposeMMKernel(MMArgs a) {
       }
 
   Fetch fa, fb;
-  auto fetchAll = [&](int k0) {
+  auto fetchAll = [&](int k0) __attribute__((always_inline)) {
     fa = fetchSlice<VEC4>(a.A, a.aRow, a.aK, a.I, i0, a.K, k0, a.XY, x0, t);
     fb = fetchSlice<VEC4>(a.B, a.bCol, a.bK, a.J, j0, a.K, k0, a.XY, x0, t);
   };
-  fetchAll(0);
+  auto stashAll = [&](int buf, int k0) __attribute__((always_inline)) {
+    float* base = lds + buf * BUF;
+    stashSlice(base, base + PLANE, fa, a.aSign, a.I, i0, a.K, k0, a.XY, x0, t);
+    stashSlice(base + 2 * PLANE, base + 3 * PLANE, fb, a.bSign, a.J, j0, a.K, k0, a.XY, x0, t);
+  };
+  // Two slice buffers, one barrier per slice: while the waves multiply slice n out
+  // of one buffer, each of them first parks slice n+1 (already in its registers) in
+  // the other and requests slice n+2.
+  if (a.K > 0) {  // with K = 0 the operands may have no memory behind them
+    fetchAll(0);
+    stashAll(0, 0);
+    if (KC < a.K) fetchAll(KC);
+  }
+  __syncthreads();
   const int xo = w * XS + lane % 32 + 64 * (lane / 32);  // bin w, row/col lane%32, k parity lane/32
-  for (int k0 = 0; k0 < a.K; k0 += KC) {
-    __syncthreads();  // previous slice fully consumed
-    stashSlice(Ar, Ai, fa, a.aSign, t);
-    stashSlice(Br, Bi, fb, a.bSign, t);
-    __syncthreads();
-    if (k0 + KC < a.K) fetchAll(k0 + KC);
+  int cur = 0;
+  for (int k0 = 0; k0 < a.K; k0 += KC, cur ^= 1) {
+    if (k0 + KC < a.K) {
+      stashAll(cur ^ 1, k0 + KC);
+      if (k0 + 2 * KC < a.K) fetchAll(k0 + 2 * KC);
+    }
+    const float* Ar = lds + cur * BUF;
+    const float* Ai = Ar + PLANE;
+    const float* Br = Ar + 2 * PLANE;
+    const float* Bi = Ar + 3 * PLANE;
 #pragma unroll
     for (int s = 0; s < KC / 2; ++s) {
       // the lane supplies row/col lane%32 (+32 for the second sub-tile) at k = 2s + lane/32
@@ -178,6 +198,7 @@ __global__ __launch_bounds__(THREADS) void transposeMMKernel(MMArgs a) {
           cim[si][sj] = __builtin_amdgcn_mfma_f32_32x32x2f32(ai[si], br[sj], cim[si][sj], 0, 0, 0);
         }
     }
+    __syncthreads();  // slice k0 consumed by everybody, slice k0 + KC parked by everybody
   }
 
   // ---- epilogue: C leaves through LDS so that every store covers whole runs (the
@@ -250,7 +271,7 @@ int launchTransposeMM(const float* A, long a0, long a1, const float* B, long b0,
   const int total = m.chunks * ceilDiv(J, TJ) * ceilDiv(I, TI);
   dim3 grid((total + 7) / 8 * 8), block(THREADS);
   const bool vec4 = aligned(A, 16) && aligned(B, 16) && a0 % 4 == 0 && a1 % 4 == 0 &&
-                    b0 % 4 == 0 && b1 % 4 == 0;
+                    b0 % 4 == 0 && b1 % 4 == 0 && XY % 2 == 0;
   if (vec4)
     transposeMMKernel<true><<<grid, block, 0, s>>>(m);
   else

@@ -35,6 +35,9 @@ ROLES = [(False, True), (True, False), (False, False)]  # updateOutput, accGrad,
     (33, 7, 5, (17, 32)),       # ragged I/J/K, xy = 544
     (1, 3, 3, (5, 8)),          # batch 1, RGB-like reduction
     (40, 70, 64, (3, 2)),       # xy = 6: partial bin chunk
+    (8, 8, 9, (3, 3)),          # odd xy (last bin has no pair), three slices with a tail
+    (16, 8, 1, (1, 5)),         # a single k
+    (70, 130, 12, (1, 13)),     # several tiles both ways, odd xy
 ])
 def test_mm_vs_oracle(oracle, conjA, conjB, I, J, K, shape):
     xy = shape[0] * shape[1]
@@ -55,6 +58,20 @@ def test_mm_vs_oracle(oracle, conjA, conjB, I, J, K, shape):
     assert rc == F.Success
     want_acc = oracle.transpose_mm(A3, B3, conjA, conjB, 0.125, C=C0.reshape(I, J, xy, 2))
     assert rel(acc.reshape(I, J, xy, 2), want_acc) < TOL_FFT
+
+
+def test_mm_empty_reduction():
+    """K = 0: C = invNorm * (accumulate ? C : 0); the operands have no elements."""
+    d = dev()
+    A = torch.zeros((4, 0, 40, 2), device=d)
+    B = torch.zeros((5, 0, 40, 2), device=d)
+    C = torch.full((4, 5, 40, 2), 3.0, device=d)
+    assert F.transposeMM(A, B, C, 0.5, False, True, True) == F.Success
+    torch.cuda.synchronize()
+    assert float((C - 1.5).abs().max()) == 0.0
+    assert F.transposeMM(A, B, C, 0.5, False, True, False) == F.Success
+    torch.cuda.synchronize()
+    assert float(C.abs().max()) == 0.0
 
 
 def test_mm_rank3_rank4_and_errors():
