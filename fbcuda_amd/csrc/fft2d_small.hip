@@ -80,6 +80,27 @@ __global__ __launch_bounds__(64) void fft2dSmallForward(RealView real, CplxView 
   auto copyOut = [&](int b0) __attribute__((always_inline)) {
     staticFor<C::ITERS>([&](auto tt) {
       constexpr int t = decltype(tt)::value;
+      // One iteration stores 64 / (N/2) consecutive spectral rows.  When none of
+      // them is row 0 or N/2 of a plane (12 of the 17 iterations at N = 32) plane and
+      // row are compile-time constants plus the lane's row within the iteration.
+      constexpr int RPI = 64 / (N / 2);
+      constexpr int R0 = RPI * t, pp0 = R0 / (H + 1), r0 = R0 % (H + 1);
+      if constexpr (r0 >= 1 && r0 + RPI - 1 <= H - 1) {
+        const int g = lane / (N / 2), xq = lane % (N / 2);
+        const float4 v = ldsLoad4(lds + pp0 * PS + (r0 + g) * RS + 2 * xq);
+        const int bo = b0 + pp0;
+        if (bo < B) {
+          if constexpr (FAST_CPLX) {
+            reinterpret_cast<float4*>(cplx.data + (size_t)bo * cplx.sb)[(r0 + g) * (N / 2) + xq] = v;
+          } else {
+            float* o = cplx.data + (size_t)bo * cplx.sb + (size_t)(r0 + g) * cplx.sr +
+                       (size_t)(2 * xq) * cplx.sc;
+            *reinterpret_cast<float2*>(o) = float2{v.x, v.y};
+            *reinterpret_cast<float2*>(o + cplx.sc) = float2{v.z, v.w};
+          }
+        }
+        return;
+      }
       const int q = lane + 64 * t;
       const int pp = q / C::F4_PER_PLANE;
       const int rem = q % C::F4_PER_PLANE;
