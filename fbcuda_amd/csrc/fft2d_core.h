@@ -64,15 +64,28 @@ template <int N>
 __device__ __forceinline__ void loadColumnsWindowPerLane(const float* src, int sy, int sx, int h,
                                                          int w, int padL, int padU, int l,
                                                          c32 (&z0)[N / 2], c32 (&z1)[N / 2]) {
-  const int x0 = 2 * l, x1 = 2 * l + 1;
-  auto fetch = [&](int y, int x) {
-    return inWindow(y, x, padU, padL, h, w)
-               ? src[(size_t)(y - padU) * sy + (size_t)(x - padL) * sx] : 0.0f;
-  };
+  const int xa = 2 * l - padL, xb = xa + 1;
+  const bool va = (unsigned)xa < (unsigned)w, vb = (unsigned)xb < (unsigned)w;
+  // element (y, xa) of the plane is pa[y * sy]; pa itself may point outside the
+  // window and is only dereferenced under the tests
+  // (global address space stated explicitly: the plane pointer comes out of a
+  // descriptor in memory, and a generic pointer would make these flat loads)
+  typedef const __attribute__((address_space(1))) float* GlobalPtr;
+  GlobalPtr pa = (GlobalPtr)(src + (long)xa * sx - (long)padU * sy);
+  GlobalPtr pb = pa + sx;
+  float ra[N], rb[N];
+  staticFor<N>([&](auto yy) {
+    constexpr int y = decltype(yy)::value;
+    const bool vy = (unsigned)(y - padU) < (unsigned)h;
+    ra[y] = 0.0f;
+    rb[y] = 0.0f;
+    if (vy && va) ra[y] = pa[(long)y * sy];
+    if (vy && vb) rb[y] = pb[(long)y * sy];
+  });
   staticFor<N / 2>([&](auto jj) {
     constexpr int j = decltype(jj)::value;
-    z0[j] = c32{fetch(2 * j, x0), fetch(2 * j + 1, x0)};
-    z1[j] = c32{fetch(2 * j, x1), fetch(2 * j + 1, x1)};
+    z0[j] = c32{ra[2 * j], ra[2 * j + 1]};
+    z1[j] = c32{rb[2 * j], rb[2 * j + 1]};
   });
 }
 
