@@ -199,40 +199,42 @@ __global__ __launch_bounds__(kThreads) void iteratedConvKernel(ConvArgs a) {
             }
           }
         } else {
+          // Row 0.  v = this lane's real-row spectrum value of a plane: the row-0 or
+          // row-N/2 half of the packed pair (x, N - x), or for x = 0 the two real
+          // values at 0 and N/2 as (re, im).  The real pair must be multiplied
+          // component by component; written as the same four multiply-adds as a
+          // complex product, with the first factor split in (re, 0) and (0, im) and
+          // the second factor's components routed accordingly, so that all lanes of
+          // the row run one instruction stream.
           const int xx = x & (H - 1);
-          const bool second = x >= H;
-          if (xx != 0) {
-            auto half = [&](const c32* p) __attribute__((always_inline)) {
-              c32 r0, rH;
-              unpack0(p[xx], p[N - xx], &r0, &rH);
-              return second ? rH : r0;
-            };
+          const bool second = x >= H, pair = xx == 0;
+          const int i1 = xx, i2 = pair ? H : N - xx;
+          auto value = [&](const c32* p) __attribute__((always_inline)) {
+            const c32 self = p[i1], other = p[i2];
+            c32 r0, rH;
+            unpack0(self, other, &r0, &rH);
+            const c32 ends = second ? c32{self.y, other.y} : c32{self.x, other.x};
+            const c32 half = second ? rH : r0;
+            return pair ? ends : half;
+          };
+          float w2x[FQ];
 #pragma unroll
-            for (int q = 0; q < FQ; ++q) wv[q] = half(ldsu + (BN + gidx + GRP * q) * PSZ);
+          for (int q = 0; q < FQ; ++q) {
+            wv[q] = value(ldsu + (BN + gidx + GRP * q) * PSZ);
+            w2x[q] = pair ? wv[q].y : wv[q].x;
+          }
 #pragma unroll
-            for (int i = 0; i < BN; ++i) {
-              const c32 av = half(ldsu + i * PSZ);
+          for (int i = 0; i < BN; ++i) {
+            const c32 av = value(ldsu + i * PSZ);
+            const float a1y = pair ? 0.0f : av.y, a2x = pair ? 0.0f : av.x;
 #pragma unroll
-              for (int q = 0; q < FQ; ++q) {
-                const c32 p = prod<CONJ>(av, wv[q]);
-                acc[i][q][nb].x += p.x;
-                acc[i][q][nb].y += p.y;
-              }
-            }
-          } else {
-            auto ends = [&](const c32* p) __attribute__((always_inline)) {
-              const c32 p0 = p[0], pH = p[H];
-              return second ? c32{p0.y, pH.y} : c32{p0.x, pH.x};
-            };
-#pragma unroll
-            for (int q = 0; q < FQ; ++q) wv[q] = ends(ldsu + (BN + gidx + GRP * q) * PSZ);
-#pragma unroll
-            for (int i = 0; i < BN; ++i) {
-              const c32 av = ends(ldsu + i * PSZ);
-#pragma unroll
-              for (int q = 0; q < FQ; ++q) {
-                acc[i][q][nb].x += av.x * wv[q].x;
-                acc[i][q][nb].y += av.y * wv[q].y;
+            for (int q = 0; q < FQ; ++q) {
+              if (CONJ) {
+                acc[i][q][nb].x += av.x * wv[q].x + a1y * wv[q].y;
+                acc[i][q][nb].y += av.y * w2x[q] - a2x * wv[q].y;
+              } else {
+                acc[i][q][nb].x += av.x * wv[q].x - a1y * wv[q].y;
+                acc[i][q][nb].y += a2x * wv[q].y + av.y * w2x[q];
               }
             }
           }
