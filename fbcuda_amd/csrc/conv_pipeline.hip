@@ -13,11 +13,11 @@
 //      a 256-lane workgroup transforms SLOTS = 512/N planes with consecutive
 //      `row` and the same k and writes each bin as one contiguous run.
 //   2. binGemmDirect:    C[bin][i][j] = invNorm * sum_k A[bin][k][i] * conj(B[bin][k][j])
-//      one workgroup = one bin x (128 x 64) tile; k-slices of A and B are
-//      contiguous in HBM and are copied verbatim into LDS by global_load_lds;
-//      4 waves x 2 MFMA 32x32x2 sub-tiles x (re, im); counters show A + B fetched
-//      from HBM exactly once (the three j-tiles of a bin share an L2: workgroup ids
-//      are remapped per XCD) and C written once with coalesced stores.
+//      one workgroup = one bin x (128 x 64) or (64 x 64) tile; k-slices of A and B
+//      are contiguous in HBM and are copied verbatim into LDS by global_load_lds;
+//      4 waves of MFMA 32x32x2 sub-tiles x (re, im); counters show A + B fetched
+//      from HBM exactly once (the tiles of a bin share an L2: workgroup ids are
+//      remapped per XCD) and C written once with coalesced stores.
 //   3. inverseBinMajor:  C[bin][i][j] -> planes, gathering runs of SLOTS
 //      consecutive j per bin, inverse transform, crop on store.
 //
@@ -183,12 +183,13 @@ struct GemmArgs {
 };
 
 // The k-slices go from HBM straight into LDS (global_load_lds, 16 bytes per lane,
-// no staging registers or LDS store instructions) through a ring of three slices:
-// slice s+2 is requested before slice s is multiplied, one barrier per slice.  A wave instruction moves 1 KiB: one k-row of A (128 complex)
-// or two k-rows of B (2 x 64 complex); LDS has exactly the HBM layout.  Requires
-// Kp % 8 == 0 with the padding rows zeroed; rows / columns beyond Ip / Jp are
-// clamped (they only feed accumulators that are never stored).
-constexpr int GJ2 = 64, GK2 = 8, ST = 3;
+// no staging registers or LDS store instructions) through a ring of three stages:
+// slice s+2 is requested before slice s is multiplied, one barrier per slice.  A
+// wave instruction moves 1 KiB: one k-row of 128 complex or two k-rows of 64
+// complex; LDS has exactly the HBM layout.  Requires Kp % 8 == 0 with the padding
+// rows zeroed; rows / columns beyond Ip / Jp are clamped (they only feed
+// accumulators that are never stored).
+constexpr int GJ2 = 64, GK2 = 8;
 
 __device__ __forceinline__ void loadToLds(const float2* src, float2* ldsWaveBase) {
   __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
