@@ -1,0 +1,61 @@
+"""The entry points allocate nothing and only enqueue kernels on the caller's
+stream, so a HIP graph can capture them.  Every replay is checked against the
+eager result, with eager work and synchronisation between replays."""
+import pytest
+import torch
+
+import fbcuda_amd as F
+from fbcuda_amd import synth
+from gpu_util import dev
+
+pytestmark = pytest.mark.gpu
+
+
+def test_graph_capture_of_the_convolution_layer_and_transforms():
+    d = dev()
+    x = synth.normal((8, 6, 27, 27), seed=30, device=d)
+    w = synth.normal((10, 6, 5, 5), seed=31, std=0.02, device=d)
+    g = synth.normal((8, 10, 23, 23), seed=32, device=d)
+    planes = synth.normal((300, 32, 32), seed=1, device=d)
+    out, gi, gw = torch.empty_like(g), torch.empty_like(x), torch.empty_like(w)
+    spec = torch.empty((300, 17, 32, 2), device=d)
+    back = torch.empty_like(planes)
+    ws = [torch.empty(F.conv_workspace(p, 8, 6, 10, 32), dtype=torch.uint8, device=d) for p in range(3)]
+
+    def run():
+        assert F.conv_fprop(x, w, out, 32, ws[0]) == F.Success
+        assert F.conv_bprop(g, w, gi, 32, ws[1]) == F.Success
+        assert F.conv_accgrad(x, g, gw, 32, ws[2], scale=0.5) == F.Success
+        assert F.fbfft2D(planes, spec) == F.Success
+        assert F.fbifft2D(spec, back) == F.Success
+
+    run()
+    torch.cuda.synchronize()
+    want = [t.clone() for t in (out, gi, gw, spec, back)]
+
+    stream = torch.cuda.Stream()
+    stream.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(stream):
+        run()  # warm-up on the capture stream
+        stream.synchronize()
+        with torch.cuda.graph(graph, stream=stream):
+            run()
+    torch.cuda.synchronize()
+
+    for rep in range(3):
+        # new inputs each time: a replay must recompute, not return stale memory
+        x.copy_(synth.normal(tuple(x.shape), seed=40 + rep, device=d))
+        planes.copy_(synth.normal(tuple(planes.shape), seed=50 + rep, device=d))
+        for t in (out, gi, gw, spec, back):
+            t.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [t.clone() for t in (out, gi, gw, spec, back)]
+        run()  # eager, same inputs
+        torch.cuda.synchronize()
+        for a, b in zip(got, (out, gi, gw, spec, back)):
+            assert bool(torch.isfinite(a).all())
+            assert torch.equal(a, b), "replay %d differs from the eager result" % rep
+    assert not torch.equal(want[0], out)  # the inputs did change
