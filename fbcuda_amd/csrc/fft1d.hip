@@ -189,6 +189,223 @@ __global__ __launch_bounds__(k1dThreads) void fft1dInverse(Row1D a) {
   }
 }
 
+// ---- N = 64 and 128 with contiguous, 16-byte aligned operands ----
+//
+// Same staging as above, but the real-input fix-up never makes a pass of its own
+// through LDS: with one lane per row (N = 64) the whole half-length transform is in
+// the lane's registers, and with two lanes per row (N = 128) the split is chosen so
+// that the fix-up pairs (k, N/2 - k) stay inside one lane - the forward transform
+// splits its outputs by parity, the inverse its inputs (E = IFFT(z even),
+// O = IFFT(z odd), x[j] = E[j] + w^j O[j], x[j + N/4] = E[j] - w^j O[j], summed on
+// the way out of LDS).  Spectra and rows then move between LDS and HBM as plain
+// 16-byte streams.
+template <int N>
+struct CfgMid {
+  static_assert(N == 64 || N == 128, "sizes with one or two lanes per row");
+  static constexpr int H = N / 2;
+  static constexpr int G = N / 64;          // lanes per row
+  static constexpr int Q = H / G;           // points per lane (32)
+  static constexpr int ROWS = k1dThreads / G;
+  static constexpr int RS = H + 1;          // LDS row stride (complex) = spectrum row length
+};
+
+template <int N>
+__global__ __launch_bounds__(k1dThreads) void fft1dMidForward(const float* __restrict__ real,
+                                                              float* __restrict__ cplx, int B) {
+  using C = CfgMid<N>;
+  constexpr int H = C::H, G = C::G, Q = C::Q, ROWS = C::ROWS, RS = C::RS;
+  __shared__ __align__(16) c32 lds[ROWS * RS];
+  __shared__ __align__(8) c32 tw[256];
+  const int t = threadIdx.x;
+  const int b0 = blockIdx.x * ROWS;
+  const int rows = min(ROWS, B - b0);
+  if constexpr (G > 1) fillTwiddles<true>(tw, t, k1dThreads);
+
+  // ---- rows -> LDS as packed complex z[j] = (x[2j], x[2j+1]), 16 bytes per load ----
+  constexpr int LOADS = ROWS * H / 2 / k1dThreads;
+  const float4* src = reinterpret_cast<const float4*>(real + (size_t)b0 * N);
+  float4 in[LOADS];
+  staticFor<LOADS>([&](auto ii) {
+    constexpr int i = decltype(ii)::value;
+    const int idx = t + k1dThreads * i;               // float4 index: row = idx / (H/2)
+    in[i] = src[min(idx, rows * (H / 2) - 1)];
+  });
+  staticFor<LOADS>([&](auto ii) {
+    constexpr int i = decltype(ii)::value;
+    const int idx = t + k1dThreads * i;
+    c32* d = lds + (idx / (H / 2)) * RS + 2 * (idx % (H / 2));
+    d[0] = c32{in[i].x, in[i].y};
+    d[1] = c32{in[i].z, in[i].w};
+  });
+  __syncthreads();
+
+  const int row = t % ROWS, g = t / ROWS;
+  c32* zrow = lds + row * RS;
+  c32 v[Q];
+  if constexpr (G == 1) {
+    splitFFT<H, 1, true>(zrow, 0, tw, v);
+    // the row is this lane's alone and is in registers: overwrite it with F[0..H]
+    realFixupForwardEmit<H>(v, [&](auto kk, c32 val) {
+      constexpr int k = decltype(kk)::value;
+      if constexpr (k == 0) {
+        zrow[0] = c32{val.x, 0.0f};
+        zrow[H] = c32{val.y, 0.0f};
+      } else {
+        zrow[k] = val;
+      }
+    });
+  } else {
+    splitFFT<H, 2, true>(zrow, g, tw, v);   // lane g: Z[2k + g]
+    __syncthreads();                        // both lanes of a row have read it
+    auto pairOut = [&](auto kp, c32 a, c32 bq) __attribute__((always_inline)) {
+      constexpr int k = decltype(kp)::value;  // bin k pairs with H-k
+      const c32 e = c32{0.5f * (a.x + bq.x), 0.5f * (a.y - bq.y)};
+      const c32 o = c32{0.5f * (a.y + bq.y), -0.5f * (a.x - bq.x)};
+      const c32 tt = mulRoot<N, k, true>(o);
+      zrow[k] = c32{e.x + tt.x, e.y + tt.y};
+      zrow[H - k] = c32{e.x - tt.x, tt.y - e.y};
+    };
+    if (g == 0) {
+      const c32 z0 = v[0];
+      zrow[0] = c32{z0.x + z0.y, 0.0f};
+      zrow[H] = c32{z0.x - z0.y, 0.0f};
+      staticFor<Q / 2 - 1>([&](auto kk) {
+        constexpr int k = decltype(kk)::value + 1;  // bins 2k and H-2k
+        pairOut(std::integral_constant<int, 2 * k>{}, v[slot<Q>(k)], v[slot<Q>(Q - k)]);
+      });
+      const c32 m = v[slot<Q>(Q / 2)];  // bin H/2
+      zrow[H / 2] = c32{m.x, -m.y};
+    } else {
+      staticFor<Q / 2>([&](auto kk) {
+        constexpr int k = decltype(kk)::value;  // bins 2k+1 and H-2k-1
+        pairOut(std::integral_constant<int, 2 * k + 1>{}, v[slot<Q>(k)], v[slot<Q>(Q - 1 - k)]);
+      });
+    }
+  }
+  __syncthreads();
+
+  // ---- spectra out: LDS and HBM hold the same [row][H+1] stream ----
+  const int total = rows * RS;  // complex values of this workgroup
+  float4* dst = reinterpret_cast<float4*>(cplx + (size_t)b0 * 2 * RS);
+  const float4* l4 = reinterpret_cast<const float4*>(lds);
+  for (int q = t; q < total / 2; q += k1dThreads) dst[q] = l4[q];
+  if ((total & 1) && t == 0)
+    reinterpret_cast<float2*>(cplx + (size_t)b0 * 2 * RS)[total - 1] = lds[total - 1];
+}
+
+template <int N>
+__global__ __launch_bounds__(k1dThreads) void fft1dMidInverse(const float* __restrict__ cplx,
+                                                              float* __restrict__ real, int B) {
+  using C = CfgMid<N>;
+  constexpr int H = C::H, G = C::G, Q = C::Q, ROWS = C::ROWS, RS = C::RS;
+  __shared__ __align__(16) c32 lds[ROWS * RS];
+  const int t = threadIdx.x;
+  const int b0 = blockIdx.x * ROWS;
+  const int rows = min(ROWS, B - b0);
+
+  // ---- spectra -> LDS, the same [row][H+1] stream in both places ----
+  const int total = rows * RS;
+  constexpr int LOADS = (ROWS * RS / 2 + k1dThreads - 1) / k1dThreads;
+  const float4* src = reinterpret_cast<const float4*>(cplx + (size_t)b0 * 2 * RS);
+  float in[4 * LOADS];  // plain floats: always promoted to registers
+  staticFor<LOADS>([&](auto ii) {
+    constexpr int i = decltype(ii)::value;
+    const float4 v = src[min(t + k1dThreads * i, max(total / 2 - 1, 0))];
+    in[4 * i] = v.x;
+    in[4 * i + 1] = v.y;
+    in[4 * i + 2] = v.z;
+    in[4 * i + 3] = v.w;
+  });
+  float4* l4 = reinterpret_cast<float4*>(lds);
+  staticFor<LOADS>([&](auto ii) {
+    constexpr int i = decltype(ii)::value;
+    const int q = t + k1dThreads * i;
+    if (q < total / 2) l4[q] = float4{in[4 * i], in[4 * i + 1], in[4 * i + 2], in[4 * i + 3]};
+  });
+  if ((total & 1) && t == 0)
+    lds[total - 1] = reinterpret_cast<const float2*>(cplx + (size_t)b0 * 2 * RS)[total - 1];
+  __syncthreads();
+
+  const int row = t % ROWS, g = t / ROWS;
+  c32* zrow = lds + row * RS;
+  float* frow = reinterpret_cast<float*>(zrow);
+  c32 zz[Q];
+  if constexpr (G == 1) {
+    // only the real parts of F[0] and F[H] reach a real result
+    realFixupInverseFetch<H>(
+        [&](auto kk) {
+          constexpr int k = decltype(kk)::value;
+          if constexpr (k == 0)
+            return c32{zrow[0].x, zrow[H].x};
+          else
+            return zrow[k];
+        },
+        zz);
+    difFFT<H, false>(zz);
+    // private row, all of it in registers: store x[2j], x[2j+1]
+    staticFor<Q>([&](auto jj) {
+      constexpr int j = decltype(jj)::value;
+      zrow[j] = zz[slot<Q>(j)];
+    });
+  } else {
+    auto pairFix = [&](auto kk, c32& zk, c32& zhk) __attribute__((always_inline)) {
+      constexpr int k = decltype(kk)::value;
+      const c32 a = zrow[k], bb = zrow[H - k];
+      const c32 e = c32{a.x + bb.x, a.y - bb.y};
+      const c32 d = c32{a.x - bb.x, a.y + bb.y};
+      const c32 o = mulRoot<N, k, false>(d);
+      zk = c32{e.x - o.y, e.y + o.x};
+      zhk = c32{e.x + o.y, o.x - e.y};
+    };
+    if (g == 0) {
+      const float f0 = zrow[0].x, fh = zrow[H].x;
+      zz[0] = c32{f0 + fh, f0 - fh};
+      staticFor<Q / 2 - 1>([&](auto mm) {
+        constexpr int k = 2 * (decltype(mm)::value + 1);  // 2, 4, ..., H/2 - 2
+        pairFix(std::integral_constant<int, k>{}, zz[k / 2], zz[(H - k) / 2]);
+      });
+      const c32 a = zrow[H / 2];
+      zz[Q / 2] = c32{2.0f * a.x, -2.0f * a.y};
+    } else {
+      staticFor<Q / 2>([&](auto mm) {
+        constexpr int k = 2 * decltype(mm)::value + 1;    // 1, 3, ..., H/2 - 1
+        pairFix(std::integral_constant<int, k>{}, zz[(k - 1) / 2], zz[(H - k - 1) / 2]);
+      });
+    }
+    difFFT<Q, false>(zz);
+    if (g == 1) {
+      staticFor<Q>([&](auto jj) {
+        constexpr int j = decltype(jj)::value;
+        zz[slot<Q>(j)] = mulRoot<H, j, false>(zz[slot<Q>(j)]);
+      });
+    }
+    __syncthreads();  // both lanes of a row have read it
+    // E as floats [0, H) of the row, w^j O as floats [H, N)
+    staticFor<Q>([&](auto jj) {
+      constexpr int j = decltype(jj)::value;
+      reinterpret_cast<c32*>(frow + H * g)[j] = zz[slot<Q>(j)];
+    });
+  }
+  __syncthreads();
+
+  // ---- rows out, 16 bytes per store ----
+  float4* dst = reinterpret_cast<float4*>(real + (size_t)b0 * N);
+  for (int q = t; q < rows * (N / 4); q += k1dThreads) {
+    const int r = q / (N / 4), c4 = q % (N / 4);
+    const float* base = reinterpret_cast<const float*>(lds + r * RS);
+    float4 o;
+    if constexpr (G == 1) {
+      o = float4{base[4 * c4], base[4 * c4 + 1], base[4 * c4 + 2], base[4 * c4 + 3]};
+    } else {
+      const int f = (4 * c4) % H;
+      const float sg = 4 * c4 < H ? 1.0f : -1.0f;
+      o = float4{base[f] + sg * base[H + f], base[f + 1] + sg * base[H + f + 1],
+                 base[f + 2] + sg * base[H + f + 2], base[f + 3] + sg * base[H + f + 3]};
+    }
+    dst[q] = o;
+  }
+}
+
 template <int N>
 int launch1d(bool forward, const Row1D& a, bool fast, hipStream_t s) {
   dim3 grid(ceilDiv(a.B, Cfg1D<N>::ROWS)), block(k1dThreads);
@@ -213,6 +430,23 @@ int launchFft1d(bool forward, int N, float* real, int sb, int sx, float* cplx, i
   if (B <= 0) return FBFFT_SUCCESS;
   Row1D a{real, sb, sx, cplx, cb, ck, B, padL};
   const bool fast = padL == 0 && sx == 1 && sb % 2 == 0 && aligned(real, 8);
+  if ((N == 64 || N == 128) && padL == 0 && sx == 1 && sb == N && ck == 2 && cb == N + 2 &&
+      aligned(real, 16) && aligned(cplx, 16)) {
+    const int rowsPerGroup = N == 64 ? CfgMid<64>::ROWS : CfgMid<128>::ROWS;
+    dim3 grid(ceilDiv(B, rowsPerGroup)), block(k1dThreads);
+    if (N == 64) {
+      if (forward)
+        fft1dMidForward<64><<<grid, block, 0, s>>>(real, cplx, B);
+      else
+        fft1dMidInverse<64><<<grid, block, 0, s>>>(cplx, real, B);
+    } else {
+      if (forward)
+        fft1dMidForward<128><<<grid, block, 0, s>>>(real, cplx, B);
+      else
+        fft1dMidInverse<128><<<grid, block, 0, s>>>(cplx, real, B);
+    }
+    return launchStatus();
+  }
   switch (N) {
     case 2: return launch1d<2>(forward, a, fast, s);
     case 4: return launch1d<4>(forward, a, fast, s);

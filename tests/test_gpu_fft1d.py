@@ -109,7 +109,7 @@ def test_strided_and_errors(oracle):
     torch.cuda.synchronize()
 
 
-@pytest.mark.parametrize("N,B", [(32, 1 << 21), (256, 1 << 18)])
+@pytest.mark.parametrize("N,B", [(32, 1 << 21), (64, (1 << 20) + 77), (128, (1 << 19) + 5), (256, 1 << 18)])
 def test_large_batch_roundtrip(N, B):
     d = dev()
     x = synth.uniform((B, N), seed=2, device=d)
