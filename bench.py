@@ -308,8 +308,8 @@ def main():
             extra["r2c_%dx%d_b%d_GBps" % (n2, n2, b2)] = round(nb / lf / 1e9, 1)
             extra["c2r_%dx%d_b%d_GBps" % (n2, n2, b2)] = round(nb / li / 1e9, 1)
             del x2, s2
-        # configs[0] (1D, 32 points, 4096 rows: launch-bound) and the largest 1D size
-        for n1, b1 in ((32, 4096), (256, 1 << 18)):
+        # configs[0] (1D, 32 points, 4096 rows: launch-bound) and the 1D sizes above one wave
+        for n1, b1 in ((32, 4096), (64, 1 << 20), (128, 1 << 19), (256, 1 << 18)):
             x1 = synth.uniform((b1, n1), seed=0, device=dev)
             s1 = torch.empty((b1, n1 // 2 + 1, 2), device=dev)
             _, lf = timed(prepared("fbfft_r2c_1d", F, x1, s1, 0), 50, 5, torch)
