@@ -221,3 +221,24 @@ def test_conv_pass_argument_checks():
     assert F.conv_accgrad(x, o, w[:, :, :2], 16, ws) == F.UnsupportedDimension
     assert F.conv_bprop(o, w, x, 16, ws[:16]) == F.UnsupportedDimension
     assert F.conv_workspace(3, 2, 3, 4, 16) == 0
+
+
+def test_conv_fprop_wide_layer(oracle):
+    """128 images x 256 output planes: enough 128-row GEMM tiles per bin (4 x 544) that the
+    pipeline keeps the 128 x 64 tile instead of the 64 x 64 one."""
+    d = dev()
+    x = synth.normal((128, 8, 27, 27), seed=60, device=d)
+    w = synth.normal((256, 8, 5, 5), seed=61, std=0.05, device=d)
+    out = torch.full((128, 256, 23, 23), float("nan"), device=d)
+    assert F.conv_fprop(x, w, out, 32, workspace(0, 128, 8, 256, 32)) == F.Success
+    torch.cuda.synchronize()
+    assert bool(torch.isfinite(out).all())
+    rng = np.random.default_rng(62)
+    coords = np.stack([rng.integers(0, 128, 4096), rng.integers(0, 256, 4096),
+                       rng.integers(0, 23, 4096), rng.integers(0, 23, 4096)], axis=1).astype(np.int32)
+    want = oracle.corr2d_valid_at(x.cpu().numpy(), w.cpu().numpy(), coords)
+    oh = out.cpu().numpy()
+    assert rel(oh[coords[:, 0], coords[:, 1], coords[:, 2], coords[:, 3]], want) < TOL_CONV
+    # whole planes at the corners of the (image, plane) grid
+    full = oracle.corr2d_valid(x.cpu().numpy()[[0, 127]], w.cpu().numpy()[[0, 255]])
+    assert rel(oh[[0, 127]][:, [0, 255]], full) < TOL_CONV
