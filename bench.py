@@ -181,6 +181,16 @@ def conv_extras(F, synth, torch, dev, extra):
     _, t = timed(tiled, 10, 2, torch)
     extra["iterated_conv_configs4_ms_per_iter"] = round(t * 1e3, 4)
     extra["iterated_conv_configs4_direct_equiv_TFLOPs"] = round(163.3e9 / t / 1e12, 1)
+    # the other two passes over the same descriptors (o4 as gradOutput)
+    for pass_, key in ((1, "bprop"), (2, "accgrad")):
+        def other():
+            rc = L.fbfft_iterated_conv(32, ctypes.c_void_p(ins.data_ptr()),
+                                       ctypes.c_void_p(outs.data_ptr()), ctypes.byref(vw4), pass_,
+                                       ctypes.c_float(1.0), 16, n, stream)
+            if rc != 1:
+                raise RuntimeError("fbfft_iterated_conv returned %d" % rc)
+        _, t = timed(other, 5, 1, torch)
+        extra["iterated_conv_configs4_%s_ms_per_iter" % key] = round(t * 1e3, 4)
 
 
 def run_only(name, steps, warmup, F, synth, torch, dev):

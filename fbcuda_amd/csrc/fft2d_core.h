@@ -148,8 +148,9 @@ __device__ __forceinline__ void columnPassInverse(const c32* plane, int l, c32 (
 }
 
 // Two columns of results through a bounds-checked strided view (crop on store).
-// ACC adds the scaled result to what the view holds instead of replacing it.
-template <int N, bool ACC = false>
+// ACC adds the scaled result to what the view holds instead of replacing it;
+// ATOMIC does that with an atomic add (several workgroups contribute to one view).
+template <int N, bool ACC = false, bool ATOMIC = false>
 __device__ __forceinline__ void storeColumnsWindow(float* dst, int sy, int sx, int h, int w, int padL,
                                                    int padU, int l, const c32 (&z0)[N / 2],
                                                    const c32 (&z1)[N / 2], float scale) {
@@ -161,7 +162,9 @@ __device__ __forceinline__ void storeColumnsWindow(float* dst, int sy, int sx, i
   float* pa = dst + (long)xa * sx;
   float* pb = dst + (long)xb * sx;
   auto put = [&](float* q, float r) __attribute__((always_inline)) {
-    if constexpr (ACC)
+    if constexpr (ATOMIC)
+      atomicAdd(q, r * scale);
+    else if constexpr (ACC)
       *q += r * scale;
     else
       *q = r * scale;

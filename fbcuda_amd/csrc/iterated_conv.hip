@@ -13,6 +13,11 @@
 //   updateGradInput  cout       outs[t](n_a, f)   weight(f, c_w)    a * w       -> ins[t](n_a, c_w)  / N^2
 //   accGradParams    tile, n    ins[t](n, c_a)    outs[t](n, f_w)   a * conj(w) -> weight(f_w, c_a) * scale / N^2
 //
+// updateOutput and updateGradInput run one workgroup per (tile, A group, W group).
+// accGradParameters reduces over all tiles and images; its reduction is also cut
+// into ranges that separate workgroups accumulate and add atomically into the
+// zeroed weight gradient, so that the chip is filled.
+//
 // The reference gives every (batch, plane) pair its own lanes and recomputes
 // both forward transforms for each of them.  Here a 512-lane workgroup owns
 // BN x FO products (8 x 8 for N = 32, 16 x 16 for N = 16, 32 x 32 for N = 8) and
@@ -24,6 +29,8 @@
 // Spectral rows 0 and N/2 travel packed as one complex row through the transforms;
 // the accumulators hold them apart.
 #include "common.h"
+
+#include <algorithm>
 #include "fft2d_core.h"
 #include "fft_regs.h"
 
@@ -40,6 +47,7 @@ struct ConvArgs {
   int wn[4];  // weight sizes: Cout, Cin, kH, kW
   int batch;
   int numTiles;
+  int splits;  // accGradParameters: workgroups along x sharing one reduction
   float scale;
 };
 
@@ -126,6 +134,11 @@ __global__ __launch_bounds__(kThreads) void iteratedConvKernel(ConvArgs a) {
   const int a0 = blockIdx.z * BN;     // first A plane (n for passes 0 and 1, c for pass 2)
   const int Cout = a.wn[0], Cin = a.wn[1];
   const int steps = PASS == 0 ? Cin : PASS == 1 ? Cout : a.numTiles * a.batch;
+  // accGradParameters reduces over every (tile, image) pair; that reduction is cut
+  // into a.splits ranges along blockIdx.x whose results meet in an atomic add
+  const int perSplit = PASS == 2 ? ((steps + a.splits - 1) / a.splits + SPI - 1) / SPI * SPI : steps;
+  const int stepBegin = PASS == 2 ? (int)blockIdx.x * perSplit : 0;
+  const int stepEnd = min(steps, stepBegin + perSplit);
 
   c32 acc[BN][FQ][NBT];
 #pragma unroll
@@ -138,7 +151,7 @@ __global__ __launch_bounds__(kThreads) void iteratedConvKernel(ConvArgs a) {
   c32* plane = lds + s * PSZ;
   // slot s transforms plane sj of reduction step SPI * it + su
   const int su = s / (BN + FO), sj = s % (BN + FO);
-  for (int it = 0; it < (steps + SPI - 1) / SPI; ++it) {
+  for (int it = stepBegin / SPI; it < (stepEnd + SPI - 1) / SPI; ++it) {
     // ---- forward transforms of this iteration's A and W planes ----
     {
       const int step = SPI * it + su;
@@ -156,7 +169,7 @@ __global__ __launch_bounds__(kThreads) void iteratedConvKernel(ConvArgs a) {
                       : tilePlane(a.outs[tl], n, w0 + sj - BN, a.batch);
       }
       c32 z0[H], z1[H];
-      if (ref.valid && step < steps) {
+      if (ref.valid && step < stepEnd) {
         loadColumnsWindowPerLane<N>(ref.p, ref.sy, ref.sx, ref.h, ref.w, ref.padL, ref.padU, l, z0,
                                     z1);
       } else {
@@ -306,11 +319,32 @@ __global__ __launch_bounds__(kThreads) void iteratedConvKernel(ConvArgs a) {
         ref = tilePlane(a.ins[tile], ai, wi, a.batch);
       else
         ref = weightPlane(a, wi, ai);
-      if (ref.valid)
-        storeColumnsWindow<N>(ref.p, ref.sy, ref.sx, ref.h, ref.w, ref.padL, ref.padU, l, z0, z1,
-                              norm);
+      if (ref.valid) {
+        if (PASS == 2 && a.splits > 1)
+          storeColumnsWindow<N, true, true>(ref.p, ref.sy, ref.sx, ref.h, ref.w, ref.padL, ref.padU,
+                                            l, z0, z1, norm);
+        else
+          storeColumnsWindow<N>(ref.p, ref.sy, ref.sx, ref.h, ref.w, ref.padL, ref.padU, l, z0, z1,
+                                norm);
+      }
     }
     __syncthreads();
+  }
+}
+
+// weight[f][c][y][x] = 0 through its strides (a fill kernel, so that the call
+// stays capturable in a graph)
+__global__ void zeroWeight(ConvArgs a) {
+  const long total = (long)a.wn[0] * a.wn[1] * a.wn[2] * a.wn[3];
+  for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (long)gridDim.x * blockDim.x) {
+    long r = i;
+    const int x = r % a.wn[3];
+    r /= a.wn[3];
+    const int y = r % a.wn[2];
+    r /= a.wn[2];
+    const int c = r % a.wn[1];
+    const int f = r / a.wn[1];
+    a.weight[(long)f * a.ws[0] + (long)c * a.ws[1] + (long)y * a.ws[2] + (long)x * a.ws[3]] = 0.0f;
   }
 }
 
@@ -325,8 +359,22 @@ int launchPass(int pass, const ConvArgs& a, hipStream_t s) {
     dim3 grid(a.numTiles, ceilDiv(Cin, C::FO), ceilDiv(a.batch, C::BN));
     iteratedConvKernel<N, 1><<<grid, kThreads, 0, s>>>(a);
   } else {
-    dim3 grid(1, ceilDiv(Cout, C::FO), ceilDiv(Cin, C::BN));
-    iteratedConvKernel<N, 2><<<grid, kThreads, 0, s>>>(a);
+    // The reference runs one block per group of planes over the whole reduction
+    // (fbfft/FFTIteratedConvolution.cuh:600-613).  With 256 CUs that leaves most of the
+    // chip idle, so the reduction is also split along x until there are about two
+    // workgroups per CU; the partial gradients are then added atomically into a
+    // zeroed weight tensor (summation order, hence the last bits, vary from run to
+    // run).  A single split stores directly.
+    ConvArgs b = a;
+    const int groups = ceilDiv(Cout, C::FO) * ceilDiv(Cin, C::BN);
+    const int steps = a.numTiles * a.batch;
+    b.splits = std::max(1, std::min(ceilDiv(512, groups), ceilDiv(steps, 2 * C::SPI)));
+    if (b.splits > 1) {
+      const long total = (long)a.wn[0] * a.wn[1] * a.wn[2] * a.wn[3];
+      zeroWeight<<<dim3((unsigned)std::min<long>((total + 255) / 256, 4096)), 256, 0, s>>>(b);
+    }
+    dim3 grid(b.splits, ceilDiv(Cout, C::FO), ceilDiv(Cin, C::BN));
+    iteratedConvKernel<N, 2><<<grid, kThreads, 0, s>>>(b);
   }
   return launchStatus();
 }
@@ -349,6 +397,7 @@ int launchIteratedConv(int N, const fbfft_tile* ins, const fbfft_tile* outs, flo
   }
   a.batch = batch;
   a.numTiles = (int)numTiles;
+  a.splits = 1;
   a.scale = scale;
   if (batch <= 0 || numTiles == 0 || wSize[0] <= 0 || wSize[1] <= 0) return 1;  // nothing to do
   int rc = N == 8 ? launchPass<8>(pass, a, s) : N == 16 ? launchPass<16>(pass, a, s)

@@ -125,7 +125,9 @@ int fbfft_transpose_mm(const fbfft_tensor* A, const fbfft_tensor* B, const fbfft
  * ins / outs are DEVICE pointers to numTiles descriptors each.  weight is
  * [Cout][Cin][kH][kW].  Returns 1 if a kernel was launched, 0 if the pass code or
  * FFT size matched nothing (the reference's bool), and a negative fbfft_error
- * (-FBFFT_HIP_ERROR ...) on launch failure. */
+ * (-FBFFT_HIP_ERROR ...) on launch failure.  FBFFT_ACC_GRAD_PARAMETERS overwrites
+ * weight with scale * gradient; partial sums of several workgroups meet in atomic
+ * adds, so its last bits can differ from run to run. */
 int fbfft_iterated_conv(int fftSize, const fbfft_tile* ins, const fbfft_tile* outs,
                         const fbfft_tensor* weight, int pass, float scale, int batchSize,
                         size_t numTiles, fbfft_stream_t stream);
