@@ -189,7 +189,7 @@ __global__ __launch_bounds__(k1dThreads) void fft1dInverse(Row1D a) {
   }
 }
 
-// ---- N = 64 and 128 with contiguous, 16-byte aligned operands ----
+// ---- N = 64, 128 and 256 with contiguous, 16-byte aligned operands ----
 //
 // Same staging as above, but the real-input fix-up never makes a pass of its own
 // through LDS: with one lane per row (N = 64) the whole half-length transform is in
@@ -197,11 +197,15 @@ __global__ __launch_bounds__(k1dThreads) void fft1dInverse(Row1D a) {
 // that the fix-up pairs (k, N/2 - k) stay inside one lane - the forward transform
 // splits its outputs by parity, the inverse its inputs (E = IFFT(z even),
 // O = IFFT(z odd), x[j] = E[j] + w^j O[j], x[j + N/4] = E[j] - w^j O[j], summed on
-// the way out of LDS).  Spectra and rows then move between LDS and HBM as plain
-// 16-byte streams.
+// the way out of LDS).  With four lanes per row (N = 256) the classes k = 0 and
+// 2 mod 4 still pair inside their lane; lanes 1 and 3 hold each other's partners:
+// forward each parks half of its transform in the row and finishes the pairs of
+// its other half, inverse each derives its own inputs from the pairs (the
+// partner's half of a pair is computed and dropped).  Spectra and rows then move between LDS and
+// HBM as plain 16-byte streams.
 template <int N>
 struct CfgMid {
-  static_assert(N == 64 || N == 128, "sizes with one or two lanes per row");
+  static_assert(N == 64 || N == 128 || N == 256, "one, two or four lanes per row");
   static constexpr int H = N / 2;
   static constexpr int G = N / 64;          // lanes per row
   static constexpr int Q = H / G;           // points per lane (32)
@@ -210,7 +214,7 @@ struct CfgMid {
 };
 
 template <int N>
-__global__ __launch_bounds__(k1dThreads) void fft1dMidForward(const float* __restrict__ real,
+__global__ __launch_bounds__(k1dThreads, 2) void fft1dMidForward(const float* __restrict__ real,
                                                               float* __restrict__ cplx, int B) {
   using C = CfgMid<N>;
   constexpr int H = C::H, G = C::G, Q = C::Q, ROWS = C::ROWS, RS = C::RS;
@@ -239,7 +243,8 @@ __global__ __launch_bounds__(k1dThreads) void fft1dMidForward(const float* __res
   });
   __syncthreads();
 
-  const int row = t % ROWS, g = t / ROWS;
+  // ROWS is a multiple of 64: g is the same for a whole wave, and says so
+  const int row = t % ROWS, g = __builtin_amdgcn_readfirstlane(t / ROWS);
   c32* zrow = lds + row * RS;
   c32 v[Q];
   if constexpr (G == 1) {
@@ -254,6 +259,60 @@ __global__ __launch_bounds__(k1dThreads) void fft1dMidForward(const float* __res
         zrow[k] = val;
       }
     });
+  } else if constexpr (G == 4) {
+    splitFFT<H, 4, true>(zrow, g, tw, v);   // lane g: Z[4k + g]; g is the wave index
+    // The results are consumed in per-wave branches below the barrier.  Without this
+    // the compiler sinks the whole transform into those branches and keeps the 128
+    // raw values it was computed from alive across the barrier instead of the 32 results.
+#pragma unroll
+    for (int j = 0; j < Q; ++j) asm volatile("" : "+v"(v[j].x), "+v"(v[j].y));
+    __syncthreads();                        // all four lanes of a row have read it
+    // F[k] and F[H-k] from a = Z[k], b = Z[H-k]
+    auto fixBoth = [&](auto kp, c32 a, c32 bq) __attribute__((always_inline)) {
+      constexpr int k = decltype(kp)::value;
+      const c32 e = c32{0.5f * (a.x + bq.x), 0.5f * (a.y - bq.y)};
+      const c32 o = c32{0.5f * (a.y + bq.y), -0.5f * (a.x - bq.x)};
+      const c32 tt = mulRoot<N, k, true>(o);
+      zrow[k] = c32{e.x + tt.x, e.y + tt.y};
+      zrow[H - k] = c32{e.x - tt.x, tt.y - e.y};
+    };
+    if (g == 0) {
+      const c32 z0 = v[0];
+      zrow[0] = c32{z0.x + z0.y, 0.0f};
+      zrow[H] = c32{z0.x - z0.y, 0.0f};
+      staticFor<Q / 2 - 1>([&](auto kk) {
+        constexpr int k = decltype(kk)::value + 1;  // bins 4k and H-4k
+        fixBoth(std::integral_constant<int, 4 * k>{}, v[slot<Q>(k)], v[slot<Q>(Q - k)]);
+      });
+      const c32 m = v[slot<Q>(Q / 2)];  // bin H/2
+      zrow[H / 2] = c32{m.x, -m.y};
+    } else if (g == 2) {
+      staticFor<Q / 2>([&](auto kk) {
+        constexpr int k = decltype(kk)::value;  // bins 4k+2 and H-4k-2
+        fixBoth(std::integral_constant<int, 4 * k + 2>{}, v[slot<Q>(k)], v[slot<Q>(Q - 1 - k)]);
+      });
+    } else {
+      // lanes 1 and 3: bin 4k+g pairs with H-4k-g = 4(Q-1-k) + (4-g), the other lane's.
+      // Each parks the upper half of its transform (k >= Q/2) at its natural positions ...
+      staticFor<Q / 2>([&](auto kk) {
+        constexpr int k = decltype(kk)::value + Q / 2;
+        zrow[4 * k + g] = v[slot<Q>(k)];
+      });
+    }
+    __syncthreads();
+    // ... and finishes the pairs of its own lower half: it alone reads and then
+    // overwrites the partner's parked values, and nobody reads its lower positions.
+    if (g == 1) {
+      staticFor<Q / 2>([&](auto kk) {
+        constexpr int k = decltype(kk)::value;
+        fixBoth(std::integral_constant<int, 4 * k + 1>{}, v[slot<Q>(k)], zrow[H - (4 * k + 1)]);
+      });
+    } else if (g == 3) {
+      staticFor<Q / 2>([&](auto kk) {
+        constexpr int k = decltype(kk)::value;
+        fixBoth(std::integral_constant<int, 4 * k + 3>{}, v[slot<Q>(k)], zrow[H - (4 * k + 3)]);
+      });
+    }
   } else {
     splitFFT<H, 2, true>(zrow, g, tw, v);   // lane g: Z[2k + g]
     __syncthreads();                        // both lanes of a row have read it
@@ -294,7 +353,7 @@ __global__ __launch_bounds__(k1dThreads) void fft1dMidForward(const float* __res
 }
 
 template <int N>
-__global__ __launch_bounds__(k1dThreads) void fft1dMidInverse(const float* __restrict__ cplx,
+__global__ __launch_bounds__(k1dThreads, 2) void fft1dMidInverse(const float* __restrict__ cplx,
                                                               float* __restrict__ real, int B) {
   using C = CfgMid<N>;
   constexpr int H = C::H, G = C::G, Q = C::Q, ROWS = C::ROWS, RS = C::RS;
@@ -326,7 +385,8 @@ __global__ __launch_bounds__(k1dThreads) void fft1dMidInverse(const float* __res
     lds[total - 1] = reinterpret_cast<const float2*>(cplx + (size_t)b0 * 2 * RS)[total - 1];
   __syncthreads();
 
-  const int row = t % ROWS, g = t / ROWS;
+  // ROWS is a multiple of 64: g is the same for a whole wave, and says so
+  const int row = t % ROWS, g = __builtin_amdgcn_readfirstlane(t / ROWS);
   c32* zrow = lds + row * RS;
   float* frow = reinterpret_cast<float*>(zrow);
   c32 zz[Q];
@@ -346,6 +406,68 @@ __global__ __launch_bounds__(k1dThreads) void fft1dMidInverse(const float* __res
     staticFor<Q>([&](auto jj) {
       constexpr int j = decltype(jj)::value;
       zrow[j] = zz[slot<Q>(j)];
+    });
+  } else if constexpr (G == 4) {
+    // lane g takes z[4m + g]; E_g = IFFT(z[4m + g]), x[j + Q q] = sum_g i^(g q) w^(g j) E_g[j]
+    auto pairFix = [&](auto kk, c32& zk, c32& zhk) __attribute__((always_inline)) {
+      constexpr int k = decltype(kk)::value;
+      const c32 a = zrow[k], bb = zrow[H - k];
+      const c32 e = c32{a.x + bb.x, a.y - bb.y};
+      const c32 d = c32{a.x - bb.x, a.y + bb.y};
+      const c32 o = mulRoot<N, k, false>(d);
+      zk = c32{e.x - o.y, e.y + o.x};
+      zhk = c32{e.x + o.y, o.x - e.y};
+    };
+    if (g == 0) {
+      const float f0 = zrow[0].x, fh = zrow[H].x;
+      zz[0] = c32{f0 + fh, f0 - fh};
+      staticFor<Q / 2 - 1>([&](auto mm) {
+        constexpr int m = decltype(mm)::value + 1;  // z[4m] and z[H - 4m] = z[4(Q - m)]
+        pairFix(std::integral_constant<int, 4 * m>{}, zz[m], zz[Q - m]);
+      });
+      const c32 a = zrow[H / 2];
+      zz[Q / 2] = c32{2.0f * a.x, -2.0f * a.y};
+    } else if (g == 2) {
+      staticFor<Q / 2>([&](auto mm) {
+        constexpr int m = decltype(mm)::value;      // z[4m+2] and z[H-4m-2] = z[4(Q-1-m)+2]
+        pairFix(std::integral_constant<int, 4 * m + 2>{}, zz[m], zz[Q - 1 - m]);
+      });
+    } else if (g == 1) {
+      staticFor<Q>([&](auto mm) {
+        constexpr int m = decltype(mm)::value;      // own z[4m+1]; the pair's other half is lane 3's
+        c32 drop;
+        pairFix(std::integral_constant<int, 4 * m + 1>{}, zz[m], drop);
+      });
+    } else {
+      staticFor<Q>([&](auto mm) {
+        constexpr int m = decltype(mm)::value;      // own z[4m+3] = z[H - k], k = 4(Q-1-m)+1
+        c32 drop;
+        pairFix(std::integral_constant<int, 4 * (Q - 1 - m) + 1>{}, drop, zz[m]);
+      });
+    }
+    difFFT<Q, false>(zz);
+    // w^(g j), w = e^(2 pi i / H); exponents of H/2 and more are the negated lower half
+    auto twist = [&](auto gg) __attribute__((always_inline)) {
+      constexpr int GG = decltype(gg)::value;
+      staticFor<Q>([&](auto jj) {
+        constexpr int j = decltype(jj)::value;
+        constexpr int ex = GG * j;
+        const c32 val = zz[slot<Q>(j)];
+        if constexpr (ex < H / 2) {
+          zz[slot<Q>(j)] = mulRoot<H, ex, false>(val);
+        } else {
+          const c32 r = mulRoot<H, ex - H / 2, false>(val);
+          zz[slot<Q>(j)] = c32{-r.x, -r.y};
+        }
+      });
+    };
+    if (g == 1) twist(std::integral_constant<int, 1>{});
+    if (g == 2) twist(std::integral_constant<int, 2>{});
+    if (g == 3) twist(std::integral_constant<int, 3>{});
+    __syncthreads();  // all four lanes of a row have read it
+    staticFor<Q>([&](auto jj) {
+      constexpr int j = decltype(jj)::value;
+      zrow[Q * g + j] = zz[slot<Q>(j)];
     });
   } else {
     auto pairFix = [&](auto kk, c32& zk, c32& zhk) __attribute__((always_inline)) {
@@ -396,6 +518,23 @@ __global__ __launch_bounds__(k1dThreads) void fft1dMidInverse(const float* __res
     float4 o;
     if constexpr (G == 1) {
       o = float4{base[4 * c4], base[4 * c4 + 1], base[4 * c4 + 2], base[4 * c4 + 3]};
+    } else if constexpr (G == 4) {
+      // complex outputs jc, jc+1 with jc = 2 c4 = j + Q q: A = T0 + (-1)^q T2,
+      // Bv = T1 + (-1)^q T3, x = A + i^q Bv
+      const int jc = 2 * c4, q4 = jc / Q, f = 2 * (jc % Q);
+      const float s2 = (q4 & 1) ? -1.0f : 1.0f;
+      float av[4], bv[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        av[e] = base[f + e] + s2 * base[2 * (2 * Q) + f + e];
+        bv[e] = base[2 * Q + f + e] + s2 * base[3 * (2 * Q) + f + e];
+      }
+      // i^q (bx, by): q=0 (bx, by), 1 (-by, bx), 2 (-bx, -by), 3 (by, -bx)
+      const bool rot = q4 & 1;
+      const float sg = (q4 == 0 || q4 == 3) ? 1.0f : -1.0f;   // sign of the first component
+      const float sh = (q4 == 0 || q4 == 1) ? 1.0f : -1.0f;   // sign of the second component
+      o = float4{av[0] + sg * (rot ? bv[1] : bv[0]), av[1] + sh * (rot ? bv[0] : bv[1]),
+                 av[2] + sg * (rot ? bv[3] : bv[2]), av[3] + sh * (rot ? bv[2] : bv[3])};
     } else {
       const int f = (4 * c4) % H;
       const float sg = 4 * c4 < H ? 1.0f : -1.0f;
@@ -430,20 +569,25 @@ int launchFft1d(bool forward, int N, float* real, int sb, int sx, float* cplx, i
   if (B <= 0) return FBFFT_SUCCESS;
   Row1D a{real, sb, sx, cplx, cb, ck, B, padL};
   const bool fast = padL == 0 && sx == 1 && sb % 2 == 0 && aligned(real, 8);
-  if ((N == 64 || N == 128) && padL == 0 && sx == 1 && sb == N && ck == 2 && cb == N + 2 &&
-      aligned(real, 16) && aligned(cplx, 16)) {
-    const int rowsPerGroup = N == 64 ? CfgMid<64>::ROWS : CfgMid<128>::ROWS;
+  if ((N == 64 || N == 128 || N == 256) && padL == 0 && sx == 1 && sb == N && ck == 2 &&
+      cb == N + 2 && aligned(real, 16) && aligned(cplx, 16)) {
+    const int rowsPerGroup = k1dThreads / (N / 64);
     dim3 grid(ceilDiv(B, rowsPerGroup)), block(k1dThreads);
     if (N == 64) {
       if (forward)
         fft1dMidForward<64><<<grid, block, 0, s>>>(real, cplx, B);
       else
         fft1dMidInverse<64><<<grid, block, 0, s>>>(cplx, real, B);
-    } else {
+    } else if (N == 128) {
       if (forward)
         fft1dMidForward<128><<<grid, block, 0, s>>>(real, cplx, B);
       else
         fft1dMidInverse<128><<<grid, block, 0, s>>>(cplx, real, B);
+    } else {
+      if (forward)
+        fft1dMidForward<256><<<grid, block, 0, s>>>(real, cplx, B);
+      else
+        fft1dMidInverse<256><<<grid, block, 0, s>>>(cplx, real, B);
     }
     return launchStatus();
   }
