@@ -206,7 +206,7 @@ struct GemmStage {
 // TI = 64 (few rows, or too few 128-row tiles to balance the chip): wave w owns rows
 // 32 (w % 2).. and columns 32 (w / 2)..
 template <int TI>
-__global__ __launch_bounds__(kT, 4) void binGemmDirect(GemmArgs g) {
+__global__ __launch_bounds__(kT, TI == 128 ? 3 : 4) void binGemmDirect(GemmArgs g) {
   static_assert(TI == 128 || TI == 64, "tile rows");
   constexpr int NQ = TI == 128 ? 2 : 1;
   constexpr int LOADS = TI == 128 ? 3 : 2;  // global->LDS instructions per wave and slice
@@ -235,13 +235,19 @@ __global__ __launch_bounds__(kT, 4) void binGemmDirect(GemmArgs g) {
   const int ia = min(i0 + 2 * (TI == 128 ? lane : lane % 32), g.Ip - 2);
   const int jb = min(j0 + 2 * (lane % 32), g.Jp - 2);
 
-  floatx16 cre[NQ], cim[NQ];
+  // Three real products per complex product instead of four: with a = ar + i ai and
+  // b = br + i bi,  a conj(b) = (k1 - k3) + i (k1 + k2)  for
+  //   k1 = (ar + ai) br,  k2 = -ar (br + bi),  k3 = ai (br - bi).
+  // The sums cost three VALU adds per operand pair; the matrix pipeline, which
+  // bounds this kernel, does a quarter less work.
+  floatx16 k1[NQ], k2[NQ], k3[NQ];
 #pragma unroll
   for (int q = 0; q < NQ; ++q)
 #pragma unroll
     for (int v = 0; v < 16; ++v) {
-      cre[q][v] = 0.f;
-      cim[q][v] = 0.f;
+      k1[q][v] = 0.f;
+      k2[q][v] = 0.f;
+      k3[q][v] = 0.f;
     }
 
   const int slices = g.Kp / GK2;
@@ -279,14 +285,14 @@ __global__ __launch_bounds__(kT, 4) void binGemmDirect(GemmArgs g) {
 #pragma unroll
     for (int s2 = 0; s2 < GK2 / 2; ++s2) {
       const float2 a = av[s2];
-      const float nar = -a.x;
+      const float as = a.x + a.y;
 #pragma unroll
       for (int q = 0; q < NQ; ++q) {
         const float2 b = bv[s2][q];
-        cre[q] = __builtin_amdgcn_mfma_f32_32x32x2f32(a.x, b.x, cre[q], 0, 0, 0);
-        cim[q] = __builtin_amdgcn_mfma_f32_32x32x2f32(a.y, b.x, cim[q], 0, 0, 0);
-        cre[q] = __builtin_amdgcn_mfma_f32_32x32x2f32(a.y, b.y, cre[q], 0, 0, 0);
-        cim[q] = __builtin_amdgcn_mfma_f32_32x32x2f32(nar, b.y, cim[q], 0, 0, 0);
+        const float nbs = -b.x - b.y, bd = b.x - b.y;
+        k1[q] = __builtin_amdgcn_mfma_f32_32x32x2f32(as, b.x, k1[q], 0, 0, 0);
+        k2[q] = __builtin_amdgcn_mfma_f32_32x32x2f32(a.x, nbs, k2[q], 0, 0, 0);
+        k3[q] = __builtin_amdgcn_mfma_f32_32x32x2f32(a.y, bd, k3[q], 0, 0, 0);
       }
     }
   };
@@ -313,7 +319,9 @@ __global__ __launch_bounds__(kT, 4) void binGemmDirect(GemmArgs g) {
 #pragma unroll
     for (int v = 0; v < 16; ++v) {
       const int i = i0 + 32 * rb + 8 * (v / 4) + 4 * h + v % 4;
-      if (i < g.I) Cb[(long)i * g.Jp + j] = float2{cre[q][v] * g.invNorm, cim[q][v] * g.invNorm};
+      if (i < g.I)
+        Cb[(long)i * g.Jp + j] =
+            float2{(k1[q][v] - k3[q][v]) * g.invNorm, (k1[q][v] + k2[q][v]) * g.invNorm};
     }
   }
 }
