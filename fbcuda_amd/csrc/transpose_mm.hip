@@ -10,15 +10,16 @@
 // are needed for every bin of a run at once, which bounds the tile: a workgroup
 // of 8 waves owns a 64 x 64 tile of C for 8 consecutive bins (64-byte runs; the
 // other half of each line goes to the neighbouring workgroup on the same XCD),
-// wave w owning bin w: 4 MFMA 32x32 sub-tiles x (re, im) = 128 accumulator
-// registers per lane.
+// wave w owning bin w: 4 MFMA 32x32 sub-tiles x 3 partial products = 192
+// accumulator registers per lane.
 //
 // Per 4-deep slice of k the workgroup stages opA and opB in LDS split into real
 // and imaginary planes [bin][k][row] (conjugation folded into the sign of the
 // imaginary plane), two buffers deep, while the slice after next is in flight in
 // registers; each
-// wave then issues v_mfma_f32_32x32x2_f32, four real products per complex
-// product: Cre += Ar*Br + (-Ai)*Bi, Cim += Ar*Bi + Ai*Br.  C leaves through LDS
+// wave then issues v_mfma_f32_32x32x2_f32, three real products per complex
+// product (k1 = (Ar+Ai) Br, k2 = Ar (Bi-Br), k3 = Ai (Br+Bi); Cre = k1 - k3,
+// Cim = k1 + k2).  C leaves through LDS
 // so that stores cover whole runs.  Only this contraction uses MFMA; it is the
 // one dense product of the convolution path.
 #include "common.h"
@@ -129,16 +130,20 @@ __global__ __launch_bounds__(THREADS) void transposeMMKernel(MMArgs a) {
   const int j0 = (rem % tilesJ) * TJ;
   const int i0 = (rem / tilesJ) * TI;
 
-  // sub-tile (si, sj): rows 32*si.., columns 32*sj..
-  floatx16 cre[2][2], cim[2][2];
+  // sub-tile (si, sj): rows 32*si.., columns 32*sj...  Three real products per complex
+  // product: with a = ar + i ai, b = br + i bi (conjugation already in the sign of
+  // the imaginary planes), a b = (k1 - k3) + i (k1 + k2) for
+  //   k1 = (ar + ai) br,  k2 = ar (bi - br),  k3 = ai (br + bi).
+  floatx16 k1[2][2], k2[2][2], k3[2][2];
 #pragma unroll
   for (int si = 0; si < 2; ++si)
 #pragma unroll
     for (int sj = 0; sj < 2; ++sj)
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
-        cre[si][sj][r] = 0.f;
-        cim[si][sj][r] = 0.f;
+        k1[si][sj][r] = 0.f;
+        k2[si][sj][r] = 0.f;
+        k3[si][sj][r] = 0.f;
       }
 
   Fetch fa, fb;
@@ -183,19 +188,20 @@ __global__ __launch_bounds__(THREADS) void transposeMMKernel(MMArgs a) {
         br[q] = Br[o + 32 * q];
         bi[q] = Bi[o + 32 * q];
       }
+      float as[2], bd[2], bs[2];
+#pragma unroll
+      for (int q = 0; q < 2; ++q) {
+        as[q] = ar[q] + ai[q];
+        bd[q] = bi[q] - br[q];
+        bs[q] = br[q] + bi[q];
+      }
 #pragma unroll
       for (int si = 0; si < 2; ++si)
 #pragma unroll
         for (int sj = 0; sj < 2; ++sj) {
-          cre[si][sj] = __builtin_amdgcn_mfma_f32_32x32x2f32(ar[si], br[sj], cre[si][sj], 0, 0, 0);
-          cim[si][sj] = __builtin_amdgcn_mfma_f32_32x32x2f32(ar[si], bi[sj], cim[si][sj], 0, 0, 0);
-        }
-#pragma unroll
-      for (int si = 0; si < 2; ++si)
-#pragma unroll
-        for (int sj = 0; sj < 2; ++sj) {
-          cre[si][sj] = __builtin_amdgcn_mfma_f32_32x32x2f32(-ai[si], bi[sj], cre[si][sj], 0, 0, 0);
-          cim[si][sj] = __builtin_amdgcn_mfma_f32_32x32x2f32(ai[si], br[sj], cim[si][sj], 0, 0, 0);
+          k1[si][sj] = __builtin_amdgcn_mfma_f32_32x32x2f32(as[si], br[sj], k1[si][sj], 0, 0, 0);
+          k2[si][sj] = __builtin_amdgcn_mfma_f32_32x32x2f32(ar[si], bd[sj], k2[si][sj], 0, 0, 0);
+          k3[si][sj] = __builtin_amdgcn_mfma_f32_32x32x2f32(ai[si], bs[sj], k3[si][sj], 0, 0, 0);
         }
     }
     __syncthreads();  // slice k0 consumed by everybody, slice k0 + KC parked by everybody
@@ -217,7 +223,8 @@ __global__ __launch_bounds__(THREADS) void transposeMMKernel(MMArgs a) {
 #pragma unroll
         for (int rr = 0; rr < 4; ++rr)
           stage[((4 * hh + rr) * TJ + 32 * sj + col) * CSTR + w] =
-              float2{cre[si][sj][4 * c + rr], cim[si][sj][4 * c + rr]};
+              float2{k1[si][sj][4 * c + rr] - k3[si][sj][4 * c + rr],
+                     k1[si][sj][4 * c + rr] + k2[si][sj][4 * c + rr]};
       __syncthreads();
       // 512 (row, col) elements x 8 bins: 8 lanes per element, 64 elements per pass
       const int xl = t % 8;
