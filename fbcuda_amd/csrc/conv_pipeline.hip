@@ -15,7 +15,8 @@
 //   2. binGemmDirect:    C[bin][i][j] = invNorm * sum_k A[bin][k][i] * conj(B[bin][k][j])
 //      one workgroup = one bin x (128 x 64) or (64 x 64) tile; k-slices of A and B
 //      are contiguous in HBM and are copied verbatim into LDS by global_load_lds;
-//      4 waves of MFMA 32x32x2 sub-tiles x (re, im); counters show A + B fetched
+//      4 waves of MFMA 32x32x2 sub-tiles, three real products per complex one;
+//      counters show A + B fetched
 //      from HBM exactly once (the tiles of a bin share an L2: workgroup ids are
 //      remapped per XCD) and C written once with coalesced stores.
 //   3. inverseBinMajor:  C[bin][i][j] -> planes, gathering runs of SLOTS
