@@ -165,6 +165,22 @@ def conv_extras(F, synth, torch, dev, extra):
     extra["transposeMM_configs3_TFLOPs"] = round(6.845e9 / t / 1e12, 1)
     extra["transposeMM_configs3_frac_of_fp32_mfma_peak"] = round(6.845e9 / t / 157.3e12, 4)
     del A, Bm, C, x, w, out, ws
+    # a 64-point layer (plane-major spectra through transposeMM): 32x32x60x60 * 64x32x5x5
+    x6 = synth.normal((32, 32, 60, 60), seed=50, device=dev)
+    w6 = synth.normal((64, 32, 5, 5), seed=51, std=0.02, device=dev)
+    o6 = torch.empty((32, 64, 56, 56), device=dev)
+    ws6 = torch.empty(F.conv_workspace(0, 32, 32, 64, 64), dtype=torch.uint8, device=dev)
+    v6 = (F.view(x6), F.view(w6), F.view(o6))
+
+    def conv64():
+        if L.fbfft_conv_fprop(ctypes.byref(v6[0]), ctypes.byref(v6[1]), ctypes.byref(v6[2]), 64,
+                              ctypes.c_void_p(ws6.data_ptr()), ws6.numel(), stream) != 0:
+            raise RuntimeError("fbfft_conv_fprop (64) failed")
+    _, t = timed(conv64, 50, 5, torch)
+    flop64 = 2.0 * 32 * 64 * 56 * 56 * 32 * 25
+    extra["fft_conv_64pt_32x32x60x60_k5_f64_ms_per_iter"] = round(t * 1e3, 4)
+    extra["fft_conv_64pt_direct_equiv_TFLOPs"] = round(flop64 / t / 1e12, 1)
+    del x6, w6, o6, ws6
     # configs[4]
     x4 = synth.uniform((16, 32, 256, 256), seed=40, device=dev)
     w4 = synth.normal((32, 32, 9, 9), seed=41, std=0.05, device=dev)

@@ -181,7 +181,7 @@ extern "C" int fbfft_transpose_mm(const fbfft_tensor* A, const fbfft_tensor* B,
 
 namespace {
 
-bool convSizeOk(int N) { return N == 8 || N == 16 || N == 32; }
+bool convSizeOk(int N) { return N == 8 || N == 16 || N == 32 || N == 64 || N == 128; }
 
 // Shapes of one convolution layer: input [B][Cin][H][W], weight [Cout][Cin][kH][kW],
 // output [B][Cout][H-kH+1][W-kW+1], H, W <= N.

@@ -73,4 +73,11 @@ int launchConvPass(int pass, int N, float* x, const int* xStride, const int* xSi
                    const int* outSize, float scale, bool accumulate, void* workspace,
                    hipStream_t s);
 
+// the same passes for 64- and 128-point transforms (conv_split.hip)
+size_t convSplitWorkspaceBytes(int pass, int N, int B, int Cin, int Cout);
+int launchConvSplit(int pass, int N, float* x, const int* xStride, const int* xSize, float* y,
+                    const int* yStride, const int* ySize, float* out, const int* outStride,
+                    const int* outSize, float scale, bool accumulate, void* workspace,
+                    hipStream_t s);
+
 }  // namespace fbfft_amd

@@ -418,6 +418,7 @@ static void passDims(int pass, int B, int Cin, int Cout, int* I, int* J, int* K)
 }
 
 size_t convWorkspaceBytes(int pass, int N, int B, int Cin, int Cout) {
+  if (N > 32) return convSplitWorkspaceBytes(pass, N, B, Cin, Cout);
   int I, J, K;
   passDims(pass, B, Cin, Cout, &I, &J, &K);
   size_t n = N == 8 ? workspaceFloat2<8>(I, J, K)
@@ -433,6 +434,9 @@ int launchConvPass(int pass, int N, float* x, const int* xStride, const int* xSi
                    const int* yStride, const int* ySize, float* out, const int* outStride,
                    const int* outSize, float scale, bool accumulate, void* workspace,
                    hipStream_t s) {
+  if (N > 32)
+    return launchConvSplit(pass, N, x, xStride, xSize, y, yStride, ySize, out, outStride, outSize,
+                           scale, accumulate, workspace, s);
   PlaneSet px, py, po;
   if (pass == 0) {
     px = planes(x, xStride, xSize, 0, 1);

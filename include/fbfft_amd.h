@@ -152,7 +152,9 @@ size_t fbfft_make_tiles(const fbfft_tensor* input, const fbfft_tensor* output, i
  * above, one entry point per pass of the role table at MM-inl.cuh:188-196.
  * Shapes throughout: input / gradInput [B][Cin][H][W], weight / gradWeight
  * [Cout][Cin][kH][kW], output / gradOutput [B][Cout][H-kH+1][W-kW+1], with
- * H, W <= fftSize in {8,16,32}.  Valid cross-correlation, no kernel flip.
+ * H, W <= fftSize in {8,16,32,64,128}.  Valid cross-correlation, no kernel flip.
+ * Sizes up to 32 hand bin-major spectra between three fused kernels; 64 and 128
+ * run fbfft2D -> transposeMM -> fbifft2D on plane-major spectra in the workspace.
  * workspace: device memory of at least fbfft_conv_workspace() bytes for that
  * pass, 256-byte aligned; its contents need not survive between calls. */
 

@@ -153,4 +153,7 @@ def test_make_tiles_capacity_and_rejects():
         F.lib().fbfft_conv_fprop_workspace(128, 64, 192, 32) > 0
     for p in (0, 1, 2):
         assert F.lib().fbfft_conv_workspace(p, 4, 5, 6, 16) % 8 == 0
-    assert F.lib().fbfft_conv_workspace(0, 4, 5, 6, 64) == 0
+    # 64 / 128: plane-major half spectra of both operands and the result
+    assert F.lib().fbfft_conv_workspace(0, 4, 5, 6, 64) == (20 + 30 + 24) * 33 * 64 * 8
+    assert F.lib().fbfft_conv_workspace(2, 4, 5, 6, 128) == (20 + 30 + 24) * 65 * 128 * 8 + 30 * 128 * 128 * 4
+    assert F.lib().fbfft_conv_workspace(0, 4, 5, 6, 256) == 0

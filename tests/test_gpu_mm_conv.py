@@ -38,6 +38,8 @@ ROLES = [(False, True), (True, False), (False, False)]  # updateOutput, accGrad,
     (8, 8, 9, (3, 3)),          # odd xy (last bin has no pair), three slices with a tail
     (16, 8, 1, (1, 5)),         # a single k
     (70, 130, 12, (1, 13)),     # several tiles both ways, odd xy
+    (9, 5, 3, (33, 64)),        # N = 64 spectra (MM-inl.cuh:778 has no instantiation for them)
+    (4, 6, 5, (65, 128)),       # N = 128 spectra
 ])
 def test_mm_vs_oracle(oracle, conjA, conjB, I, J, K, shape):
     xy = shape[0] * shape[1]
@@ -118,7 +120,8 @@ def conv(x, w, N):
 
 
 @pytest.mark.parametrize("N,H,W,k,Bn,Cin,Cout", [
-    (8, 8, 8, 3, 2, 3, 4), (16, 13, 16, 5, 3, 5, 7), (32, 27, 27, 5, 4, 8, 6), (32, 32, 30, 1, 2, 2, 2)])
+    (8, 8, 8, 3, 2, 3, 4), (16, 13, 16, 5, 3, 5, 7), (32, 27, 27, 5, 4, 8, 6), (32, 32, 30, 1, 2, 2, 2),
+    (64, 60, 57, 5, 3, 5, 4), (64, 64, 64, 11, 1, 3, 6), (128, 100, 128, 7, 2, 3, 2)])
 def test_conv_fprop_small(oracle, N, H, W, k, Bn, Cin, Cout):
     x = synth.normal((Bn, Cin, H, W), seed=30).numpy()
     w = synth.normal((Cout, Cin, k, k), seed=31, std=0.02).numpy()
@@ -150,7 +153,9 @@ def test_conv_fprop_config3(oracle):
 
 
 SHAPES = [(8, 8, 8, 3, 2, 3, 4), (16, 13, 16, 5, 3, 5, 7), (32, 27, 27, 5, 4, 8, 6),
-          (32, 32, 30, 1, 2, 2, 2), (32, 20, 31, 7, 5, 150, 9), (16, 16, 16, 3, 70, 3, 140)]
+          (32, 32, 30, 1, 2, 2, 2), (32, 20, 31, 7, 5, 150, 9), (16, 16, 16, 3, 70, 3, 140),
+          # 64- and 128-point transforms: plane-major spectra through transposeMM
+          (64, 60, 57, 5, 3, 5, 4), (64, 64, 64, 11, 1, 3, 6), (128, 100, 128, 7, 2, 3, 2)]
 
 
 def workspace(pass_, Bn, Cin, Cout, N):
@@ -216,7 +221,8 @@ def test_conv_pass_argument_checks():
     o = torch.zeros(2, 4, 14, 14, device=d)
     ws = workspace(1, 2, 3, 4, 16)
     assert F.conv_bprop(o, w, x, 16, ws) == F.Success
-    assert F.conv_bprop(o, w, x, 64, ws) == F.UnsupportedSize
+    assert F.conv_bprop(o, w, x, 256, ws) == F.UnsupportedSize
+    assert F.conv_bprop(o, w, x, 64, ws[:4096]) == F.UnsupportedDimension   # workspace too small
     assert F.conv_bprop(o[:, :3], w, x, 16, ws) == F.UnsupportedDimension
     assert F.conv_accgrad(x, o, w[:, :, :2], 16, ws) == F.UnsupportedDimension
     assert F.conv_bprop(o, w, x, 16, ws[:16]) == F.UnsupportedDimension
@@ -242,3 +248,28 @@ def test_conv_fprop_wide_layer(oracle):
     # whole planes at the corners of the (image, plane) grid
     full = oracle.corr2d_valid(x.cpu().numpy()[[0, 127]], w.cpu().numpy()[[0, 255]])
     assert rel(oh[[0, 127]][:, [0, 255]], full) < TOL_CONV
+
+
+def test_conv_split_path_strided_operands(oracle):
+    """64-point layer on views whose planes do not collapse into one batch (one
+    transform launch per image) and an accumulating weight gradient through a view."""
+    d = dev()
+    Bn, Cin, Cout, H, W, k = 3, 4, 5, 50, 64, 9
+    xbig = synth.normal((Bn, Cin + 2, H, W), seed=70, device=d)
+    x = xbig[:, 1:1 + Cin]
+    w = synth.normal((Cout, Cin, k, k), seed=71, std=0.05, device=d)
+    out = torch.full((Bn, Cout, H - k + 1, W - k + 1), float("nan"), device=d)
+    assert F.conv_fprop(x, w, out, 64, workspace(0, Bn, Cin, Cout, 64)) == F.Success
+    torch.cuda.synchronize()
+    xh, wh = x.cpu().numpy().copy(), w.cpu().numpy()
+    assert rel(out.cpu().numpy(), oracle.corr2d_valid(xh, wh)) < TOL_CONV
+    go = synth.normal(tuple(out.shape), seed=72, device=d)
+    gwbig = synth.normal((Cout, Cin, k + 3, k + 1), seed=73, device=d)
+    gw0 = gwbig.cpu().numpy().copy()
+    gw = gwbig[:, :, 2:2 + k, 1:1 + k]
+    assert F.conv_accgrad(x, go, gw, 64, workspace(2, Bn, Cin, Cout, 64), scale=0.5,
+                          accumulate=True) == F.Success
+    torch.cuda.synchronize()
+    want = gw0.copy()
+    want[:, :, 2:2 + k, 1:1 + k] += 0.5 * oracle.corr2d_grad_weight(xh, go.cpu().numpy(), k, k)
+    assert rel(gwbig.cpu().numpy(), want) < TOL_CONV
