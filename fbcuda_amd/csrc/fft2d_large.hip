@@ -78,12 +78,37 @@ __global__ __launch_bounds__(LargeCfg<N>::THREADS) void fft2dLargeForward(RealVi
       }
     });
   } else {
+    // Windowed plane (implicit zero padding, any strides): a lane keeps its column
+    // and walks down the rows.  Loads go out in batches of 16 at addresses clamped
+    // into the window, with no branch between them, and samples outside the window
+    // are zeroed when they are parked in LDS; batches below the window's last row
+    // load nothing.
     const float* src = real.data + (size_t)b * real.sb;
-    for (int q = t; q < N * N; q += THREADS) {
-      const int y = q / N, x = q % N;
-      buf[y * RSI + x] = inWindow(y, x, padU, padL, real.h, real.w)
-                             ? src[(size_t)(y - padU) * real.sy + (size_t)(x - padL) * real.sx]
-                             : 0.0f;
+    constexpr int RPI = THREADS / N;   // rows per step of the walk
+    constexpr int BATCH = 16;
+    const int x = t % N, yb = t / N;
+    const int xs = x - padL;
+    const bool xin = (unsigned)xs < (unsigned)real.w;
+    const float* colp = src + (size_t)min(max(xs, 0), real.w - 1) * real.sx;
+    const int yEnd = min(N, padU + real.h);
+#pragma unroll
+    for (int i0 = 0; i0 < N / RPI; i0 += BATCH) {
+      if (i0 * RPI < yEnd) {
+        float v[BATCH];
+#pragma unroll
+        for (int j = 0; j < BATCH; ++j) {
+          const int ys = min(max(yb + RPI * (i0 + j) - padU, 0), real.h - 1);
+          v[j] = colp[(size_t)ys * real.sy];
+        }
+#pragma unroll
+        for (int j = 0; j < BATCH; ++j) {
+          const int y = yb + RPI * (i0 + j);
+          buf[y * RSI + x] = (xin && (unsigned)(y - padU) < (unsigned)real.h) ? v[j] : 0.0f;
+        }
+      } else {
+#pragma unroll
+        for (int j = 0; j < BATCH; ++j) buf[(yb + RPI * (i0 + j)) * RSI + x] = 0.0f;
+      }
     }
   }
   __syncthreads();
@@ -283,11 +308,15 @@ __global__ __launch_bounds__(LargeCfg<N>::THREADS) void fft2dLargeInverse(CplxVi
         dst[(size_t)y * rs4 + x4] = *reinterpret_cast<const float4*>(buf + y * RSF + 4 * x4);
       });
     } else {
-      float* dst = real.data + (size_t)b * real.sb;
-      for (int q = t; q < N * N; q += THREADS) {
-        const int y = q / N, x = q % N;
-        if (inWindow(y, x, padU, padL, real.h, real.w))
-          dst[(size_t)(y - padU) * real.sy + (size_t)(x - padL) * real.sx] = buf[y * RSF + x];
+      // a lane keeps its column and walks down the rows of the window
+      constexpr int RPI = THREADS / N;
+      const int x = t % N, xs = x - padL;
+      if ((unsigned)xs < (unsigned)real.w) {
+        float* colp = real.data + (size_t)b * real.sb + (size_t)xs * real.sx;
+        const int yEnd = min(N, padU + real.h);
+#pragma unroll 8
+        for (int y = padU + t / N; y < yEnd; y += RPI)
+          colp[(size_t)(y - padU) * real.sy] = buf[y * RSF + x];
       }
     }
   } else {
@@ -365,13 +394,17 @@ __global__ __launch_bounds__(LargeCfg<N>::THREADS) void fft2dLargeInverse(CplxVi
             float4{e.x + sg * w.x, e.y + sg * w.y, e.z + sg * w.z, e.w + sg * w.w};
       });
     } else {
-      float* dst = real.data + (size_t)b * real.sb;
-      for (int q = t; q < N * N; q += THREADS) {
-        const int yy = q / N, x = q % N;
-        if (inWindow(yy, x, padU, padL, real.h, real.w)) {
-          const float e = buf[yy * RSF + x % H], w = buf[yy * RSF + H + x % H];
-          dst[(size_t)(yy - padU) * real.sy + (size_t)(x - padL) * real.sx] = x < H ? e + w : e - w;
-        }
+      // a lane keeps its column and walks down the rows of the window
+      constexpr int RPI = THREADS / N;
+      const int x = t % N, xs = x - padL;
+      if ((unsigned)xs < (unsigned)real.w) {
+        float* colp = real.data + (size_t)b * real.sb + (size_t)xs * real.sx;
+        const int yEnd = min(N, padU + real.h);
+        const float sg = x < H ? 1.0f : -1.0f;
+        const float* e = buf + x % H;
+#pragma unroll 8
+        for (int yy = padU + t / N; yy < yEnd; yy += RPI)
+          colp[(size_t)(yy - padU) * real.sy] = e[yy * RSF] + sg * e[yy * RSF + H];
       }
     }
   }
