@@ -42,11 +42,26 @@ __device__ __forceinline__ void loadColumnsWindow(const float* src, int sy, int 
   const float* pa = src + (long)min(max(xa, 0), w - 1) * sx;
   const float* pb = src + (long)min(max(xb, 0), w - 1) * sx;
   float ra[N], rb[N];
-  staticFor<N>([&](auto yy) {
-    constexpr int y = decltype(yy)::value;
-    const long oy = (long)min(max(y - padU, 0), h - 1) * sy;
-    ra[y] = pa[oy];
-    rb[y] = pb[oy];
+  // rows in batches of 8: a batch that lies wholly below the window (the same for
+  // every lane) issues no loads - a 5 x 5 filter plane costs 16 loads, not 2N
+  const int yEnd = padU + h;
+  staticFor<(N + 7) / 8>([&](auto bb) {
+    constexpr int y0 = 8 * decltype(bb)::value;
+    constexpr int y1 = y0 + 8 < N ? y0 + 8 : N;
+    if (y0 < yEnd) {
+      staticFor<y1 - y0>([&](auto yy) {
+        constexpr int y = y0 + decltype(yy)::value;
+        const long oy = (long)min(max(y - padU, 0), h - 1) * sy;
+        ra[y] = pa[oy];
+        rb[y] = pb[oy];
+      });
+    } else {
+      staticFor<y1 - y0>([&](auto yy) {
+        constexpr int y = y0 + decltype(yy)::value;
+        ra[y] = 0.0f;
+        rb[y] = 0.0f;
+      });
+    }
   });
   staticFor<N / 2>([&](auto jj) {
     constexpr int j = decltype(jj)::value;
