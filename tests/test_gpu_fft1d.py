@@ -119,3 +119,45 @@ def test_large_batch_roundtrip(N, B):
     assert F.fbifft1D(back, spec) == F.Success
     torch.cuda.synchronize()
     assert float((back / N - x).double().norm() / x.double().norm()) < TOL_FFT
+
+
+@pytest.mark.parametrize("seed", range(30))
+def test_random_batches_pads_and_views(oracle, seed):
+    """Seeded random draw over size, batch (odd tails), padL and memory layout of
+    both operands; forward against the transcription and the fp64 DFT of the
+    shifted row, inverse against the transcription (sentinel where it writes nothing)."""
+    rng = np.random.default_rng(2000 + seed)
+    N = int(rng.choice(SIZES))
+    B = int(rng.integers(1, 600))
+    padL = int(rng.integers(0, N // 2 + 1)) if rng.random() < 0.4 else 0
+    x = synth.uniform((B, N), seed=seed).numpy()
+    d = dev()
+    kind = int(rng.integers(0, 3))
+    if kind == 0:
+        real = torch.from_numpy(x).to(d)
+    elif kind == 1:                                    # padded batch stride
+        big = torch.zeros((B, N + 6), device=d)
+        real = big[:, 4:N + 4]
+        real.copy_(torch.from_numpy(x))
+    else:                                              # rows along the slow axis
+        real = torch.from_numpy(np.ascontiguousarray(x.T)).to(d).t()
+    if rng.random() < 0.5:
+        spec = torch.full((B, N // 2 + 1, 2), float("nan"), device=d)
+    else:
+        wide = torch.full((B, N // 2 + 3, 2), float("nan"), device=d)
+        spec = wide[:, 1:N // 2 + 2, :]
+    assert F.fbfft1D(real, spec, padL) == F.Success
+    torch.cuda.synchronize()
+    _, want = oracle.fbfft1d(x, padL)
+    got = spec.cpu().numpy()
+    assert rel(got, want) < TOL_FFT, (N, B, padL, kind)
+    shifted = np.zeros_like(x)
+    shifted[:, padL:] = x[:, :N - padL]
+    assert rel(got, oracle.dft1d_r2c(shifted)) < TOL_FFT
+    back = torch.full_like(real, 777.0)
+    assert F.fbifft1D(back, spec, padL) == F.Success
+    torch.cuda.synchronize()
+    _, back32 = oracle.fbifft1d(want, padL, out=np.full((B, N), 777.0, np.float32))
+    bh = back.cpu().numpy()
+    assert np.array_equal(bh == 777.0, back32 == 777.0), (N, B, padL, kind)
+    assert rel(bh, back32) < TOL_FFT, (N, B, padL, kind)

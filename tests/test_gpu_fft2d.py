@@ -182,3 +182,45 @@ def test_warp_kernel_sizes(oracle, N, B):
     torch.cuda.synchronize()
     assert rel(spec.cpu().numpy(), oracle.dft2d_r2c(x, N)) < TOL_FFT
     assert bool(torch.isnan(wide[:, 0]).all()) and bool(torch.isnan(wide[:, :, N]).all())
+
+
+@pytest.mark.parametrize("seed", range(40))
+def test_random_windows_and_views(oracle, seed):
+    """Seeded random draw over size, batch, window, padding (also windows that
+    hang over the right / bottom edge, which MemoryAccess.cuh:19-25 clips), and
+    views that are transposed or padded in memory."""
+    rng = np.random.default_rng(1000 + seed)
+    N = int(rng.choice([2, 4, 8, 16, 32, 64, 128]))
+    B = int(rng.integers(1, 20))
+    h, w = int(rng.integers(1, N + 1)), int(rng.integers(1, N + 1))
+    padL, padU = (int(rng.integers(0, N // 2 + 1)), int(rng.integers(0, N // 2 + 1))) \
+        if rng.random() < 0.6 else (0, 0)
+    x = synth.normal((B, h, w), seed=seed).numpy()
+    d = dev()
+    kind = int(rng.integers(0, 3))
+    if kind == 0:                                   # contiguous
+        real = torch.from_numpy(x).to(d)
+    elif kind == 1:                                 # padded rows and batch stride
+        big = torch.zeros((B, h + 2, w + 3), device=d)
+        real = big[:, 1:h + 1, 2:w + 2]
+        real.copy_(torch.from_numpy(x))
+    else:                                           # x and y swapped in memory
+        real = torch.from_numpy(np.ascontiguousarray(x.transpose(0, 2, 1))).to(d).transpose(1, 2)
+    if rng.random() < 0.5:
+        spec = torch.full((B, N // 2 + 1, N, 2), float("nan"), device=d)
+    else:
+        wide = torch.full((B + 1, N // 2 + 2, N + 1, 2), float("nan"), device=d)
+        spec = wide[1:, 1:, :N, :]
+    assert F.fbfft2D(real, spec, padL, padU) == F.Success
+    torch.cuda.synchronize()
+    _, want32 = oracle.fbfft2d(x, N, padL, padU)
+    got = spec.cpu().numpy()
+    assert rel(got, want32) < TOL_FFT, (N, B, h, w, padL, padU, kind)
+    assert rel(got, oracle.dft2d_r2c(x, N, padL, padU)) < TOL_FFT
+    # and back into a view of the same geometry
+    # (cells of the window that hang over the edge keep what they held)
+    back = torch.full_like(real, 7.0)
+    assert F.fbifft2D(spec, back, padL, padU) == F.Success
+    torch.cuda.synchronize()
+    _, back32 = oracle.fbifft2d(want32, h, w, padL, padU, out=np.full((B, h, w), 7.0, np.float32))
+    assert rel(back.cpu().numpy(), back32) < TOL_FFT, (N, B, h, w, padL, padU, kind)

@@ -273,3 +273,30 @@ def test_conv_split_path_strided_operands(oracle):
     want = gw0.copy()
     want[:, :, 2:2 + k, 1:1 + k] += 0.5 * oracle.corr2d_grad_weight(xh, go.cpu().numpy(), k, k)
     assert rel(gwbig.cpu().numpy(), want) < TOL_CONV
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_mm_random_shapes_and_views(oracle, seed):
+    """Seeded random draw over I, J, K, the bin count, the role and accumulation,
+    with operands that are views into larger buffers (padded leading strides)."""
+    rng = np.random.default_rng(3000 + seed)
+    I, J, K = (int(v) for v in rng.integers(1, 140, 3))
+    shape = (int(rng.integers(1, 10)), int(rng.integers(1, 20)))
+    xy = shape[0] * shape[1]
+    conjA, conjB = ROLES[int(rng.integers(0, 3))]
+    acc = bool(rng.integers(0, 2))
+    d = dev()
+
+    def operand(d0, d1, s):
+        full = synth.normal((d0 + 1, d1 + 2) + shape + (2,), seed=s, device=d)
+        return full[1:, 1:d1 + 1]                      # leading strides larger than the extents
+    A = operand(*((K, I) if conjA else (I, K)), 1 + seed)
+    B = operand(*((J, K) if conjB else (K, J)), 2 + seed)
+    C = operand(I, J, 3 + seed)
+    C0 = C.cpu().numpy().copy()
+    assert F.transposeMM(A, B, C, 0.5, conjA, conjB, acc) == F.Success
+    torch.cuda.synchronize()
+    A3 = A.cpu().numpy().reshape(A.shape[0], A.shape[1], xy, 2)
+    B3 = B.cpu().numpy().reshape(B.shape[0], B.shape[1], xy, 2)
+    want = oracle.transpose_mm(A3, B3, conjA, conjB, 0.5, C=C0.reshape(I, J, xy, 2) if acc else None)
+    assert rel(C.cpu().numpy().reshape(I, J, xy, 2), want) < TOL_FFT, (I, J, K, shape, conjA, conjB, acc)
