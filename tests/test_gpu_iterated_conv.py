@@ -164,3 +164,30 @@ def test_library_tile_grid_matches_reference_tiling(oracle):
     assert F.FFTIteratedConvolution(N, ins, outs, w, F.FFT_UpdateOutput, 1.0, Nb, n)
     torch.cuda.synchronize()
     assert rel(out.cpu().numpy(), oracle.corr2d_valid(x.cpu().numpy(), w.cpu().numpy())) < TOL_CONV
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_random_tilings(oracle, seed):
+    """updateOutput and accGradParameters on a seeded random image / filter / plane
+    count with the library's own tile grid, against fp64 direct correlation."""
+    rng = np.random.default_rng(5000 + seed)
+    N = int(rng.choice([8, 16, 32]))
+    k = int(rng.integers(1, min(N - 1, 9) + 1))
+    H, W = int(rng.integers(k, 3 * N)), int(rng.integers(k, 3 * N))
+    Nb, Cin, Cout = int(rng.integers(1, 20)), int(rng.integers(1, 12)), int(rng.integers(1, 20))
+    d = dev()
+    x = synth.uniform((Nb, Cin, H, W), seed=seed, device=d)
+    w = synth.normal((Cout, Cin, k, k), seed=seed + 1, std=0.05, device=d)
+    out = torch.full((Nb, Cout, H - k + 1, W - k + 1), float("nan"), device=d)
+    ins, outs, n = F.make_tile_grid(x, out, k, k, N)
+    tag = (N, k, H, W, Nb, Cin, Cout, n)
+    assert F.FFTIteratedConvolution(N, ins, outs, w, F.FFT_UpdateOutput, 1.0, Nb, n), tag
+    torch.cuda.synchronize()
+    xh, wh = x.cpu().numpy(), w.cpu().numpy()
+    assert rel(out.cpu().numpy(), oracle.corr2d_valid(xh, wh)) < TOL_CONV, tag
+    g = synth.normal(tuple(out.shape), seed=seed + 2, device=d)
+    gins, gouts, n2 = F.make_tile_grid(x, g, k, k, N)
+    gw = torch.full_like(w, float("nan"))
+    assert F.FFTIteratedConvolution(N, gins, gouts, gw, F.FFT_AccGradParameters, 0.25, Nb, n2), tag
+    torch.cuda.synchronize()
+    assert rel(gw.cpu().numpy(), 0.25 * oracle.corr2d_grad_weight(xh, g.cpu().numpy(), k, k)) < TOL_CONV, tag

@@ -300,3 +300,34 @@ def test_mm_random_shapes_and_views(oracle, seed):
     B3 = B.cpu().numpy().reshape(B.shape[0], B.shape[1], xy, 2)
     want = oracle.transpose_mm(A3, B3, conjA, conjB, 0.5, C=C0.reshape(I, J, xy, 2) if acc else None)
     assert rel(C.cpu().numpy().reshape(I, J, xy, 2), want) < TOL_FFT, (I, J, K, shape, conjA, conjB, acc)
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_conv_layer_random_shapes(oracle, seed):
+    """All three passes on a seeded random layer (FFT size, image and filter
+    extents, plane counts), the input being a channel slice of a larger tensor."""
+    rng = np.random.default_rng(4000 + seed)
+    N = int(rng.choice([8, 16, 32, 64, 128], p=[0.2, 0.25, 0.3, 0.15, 0.1]))
+    H, W = int(rng.integers(max(2, N // 2), N + 1)), int(rng.integers(max(2, N // 2), N + 1))
+    kH, kW = int(rng.integers(1, min(H, 9) + 1)), int(rng.integers(1, min(W, 9) + 1))
+    Bn, Cin, Cout = int(rng.integers(1, 9)), int(rng.integers(1, 12)), int(rng.integers(1, 12))
+    if N >= 64:
+        Bn, Cin, Cout = min(Bn, 3), min(Cin, 4), min(Cout, 4)
+    d = dev()
+    xbig = synth.normal((Bn, Cin + 1, H, W), seed=seed, device=d)
+    x = xbig[:, 1:]
+    w = synth.normal((Cout, Cin, kH, kW), seed=seed + 100, std=0.1, device=d)
+    go = synth.normal((Bn, Cout, H - kH + 1, W - kW + 1), seed=seed + 200, device=d)
+    tag = (N, H, W, kH, kW, Bn, Cin, Cout)
+    xh, wh, gh = x.cpu().numpy().copy(), w.cpu().numpy(), go.cpu().numpy()
+
+    out = torch.full_like(go, float("nan"))
+    assert F.conv_fprop(x, w, out, N, workspace(0, Bn, Cin, Cout, N)) == F.Success
+    gi = torch.full((Bn, Cin, H, W), float("nan"), device=d)
+    assert F.conv_bprop(go, w, gi, N, workspace(1, Bn, Cin, Cout, N)) == F.Success
+    gw = torch.full_like(w, float("nan"))
+    assert F.conv_accgrad(x, go, gw, N, workspace(2, Bn, Cin, Cout, N), scale=2.0) == F.Success
+    torch.cuda.synchronize()
+    assert rel(out.cpu().numpy(), oracle.corr2d_valid(xh, wh)) < TOL_CONV, tag
+    assert rel(gi.cpu().numpy(), oracle.corr2d_grad_input(gh, wh, H, W)) < TOL_CONV, tag
+    assert rel(gw.cpu().numpy(), 2.0 * oracle.corr2d_grad_weight(xh, gh, kH, kW)) < TOL_CONV, tag
