@@ -84,13 +84,51 @@ __global__ __launch_bounds__(LargeCfg<N>::THREADS) void fft2dLargeForward(RealVi
     // are zeroed when they are parked in LDS; batches below the window's last row
     // load nothing.
     const float* src = real.data + (size_t)b * real.sb;
+    const int yEnd = min(N, padU + real.h);
+    // rows that start on 16-byte boundaries and a window whose left edge and width are
+    // multiples of 4 (contiguous 60 x 60 planes, say) move as float4 the same way
+    const bool vec = real.sx == 1 && ((real.sy | real.sb | padL | real.w) & 3) == 0 &&
+                     (reinterpret_cast<uintptr_t>(real.data) & 15) == 0;
+    if (vec) {
+      constexpr int GPR = N / 4;           // float4 per row
+      constexpr int RPI4 = THREADS / GPR;  // rows per step
+      constexpr int STEPS = N / RPI4;      // 16
+      constexpr int HALF = STEPS / 2;
+      const int xg = t % GPR, yb = t / GPR;
+      const int xs = 4 * xg - padL;
+      const bool xin = (unsigned)xs < (unsigned)real.w;
+      const float* colp = src + min(max(xs, 0), real.w - 4);
+#pragma unroll
+      for (int j0 = 0; j0 < STEPS; j0 += HALF) {
+        float4 v[HALF];
+        if (j0 * RPI4 < yEnd) {
+#pragma unroll
+          for (int j = 0; j < HALF; ++j) {
+            const int ys = min(max(yb + RPI4 * (j0 + j) - padU, 0), real.h - 1);
+            v[j] = *reinterpret_cast<const float4*>(colp + (size_t)ys * real.sy);
+          }
+        }
+#pragma unroll
+        for (int j = 0; j < HALF; ++j) {
+          const int y = yb + RPI4 * (j0 + j);
+          const bool ok = j0 * RPI4 < yEnd && xin && (unsigned)(y - padU) < (unsigned)real.h;
+          const float4 o = ok ? v[j] : float4{0.f, 0.f, 0.f, 0.f};
+          float* d = buf + y * RSI + 4 * xg;
+          if constexpr (RSI % 4 == 0) {
+            *reinterpret_cast<float4*>(d) = o;
+          } else {
+            *reinterpret_cast<float2*>(d) = float2{o.x, o.y};
+            *reinterpret_cast<float2*>(d + 2) = float2{o.z, o.w};
+          }
+        }
+      }
+    } else {
     constexpr int RPI = THREADS / N;   // rows per step of the walk
     constexpr int BATCH = 16;
     const int x = t % N, yb = t / N;
     const int xs = x - padL;
     const bool xin = (unsigned)xs < (unsigned)real.w;
     const float* colp = src + (size_t)min(max(xs, 0), real.w - 1) * real.sx;
-    const int yEnd = min(N, padU + real.h);
 #pragma unroll
     for (int i0 = 0; i0 < N / RPI; i0 += BATCH) {
       if (i0 * RPI < yEnd) {
@@ -109,6 +147,7 @@ __global__ __launch_bounds__(LargeCfg<N>::THREADS) void fft2dLargeForward(RealVi
 #pragma unroll
         for (int j = 0; j < BATCH; ++j) buf[(yb + RPI * (i0 + j)) * RSI + x] = 0.0f;
       }
+    }
     }
   }
   __syncthreads();

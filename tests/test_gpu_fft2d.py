@@ -224,3 +224,19 @@ def test_random_windows_and_views(oracle, seed):
     torch.cuda.synchronize()
     _, back32 = oracle.fbifft2d(want32, h, w, padL, padU, out=np.full((B, h, w), 7.0, np.float32))
     assert rel(back.cpu().numpy(), back32) < TOL_FFT, (N, B, h, w, padL, padU, kind)
+
+
+@pytest.mark.parametrize("N,h,w,padL,padU", [
+    (64, 60, 60, 0, 0), (64, 60, 60, 4, 3), (64, 17, 8, 8, 40), (64, 64, 64, 4, 1),
+    (128, 124, 124, 0, 0), (128, 124, 120, 4, 2), (128, 31, 64, 60, 100), (128, 5, 4, 124, 0)])
+def test_windows_that_move_as_16_byte_words(oracle, N, h, w, padL, padU):
+    """Windows whose rows start on 16-byte boundaries with width and left edge
+    multiples of 4 take the float4 loader of the 64 / 128 kernels (also hanging
+    over the right edge)."""
+    B = 5
+    x = synth.normal((B, h, w), seed=N + h).numpy()
+    rc, got = fft2d(x, N, padL, padU)
+    assert rc == F.Success
+    _, want32 = oracle.fbfft2d(x, N, padL, padU)
+    assert rel(got, want32) < TOL_FFT
+    assert rel(got, oracle.dft2d_r2c(x, N, padL, padU)) < TOL_FFT
