@@ -86,6 +86,29 @@ __device__ __forceinline__ void loadColumnsWindowPerLane(const float* src, int s
   // (global address space stated explicitly: the plane pointer comes out of a
   // descriptor in memory, and a generic pointer would make these flat loads)
   typedef const __attribute__((address_space(1))) float* GlobalPtr;
+  // When every lane of the wave sees rows that start on 8-byte boundaries and a
+  // window whose left edge and width are even, its two columns are one 8-byte word
+  // per row, inside or outside the window together.
+  const bool pairs = sx == 1 && ((sy | padL | w) & 1) == 0 &&
+                     (reinterpret_cast<uintptr_t>(src) & 7) == 0;
+  if (__builtin_amdgcn_ballot_w64(!pairs) == 0) {
+    typedef float Pair __attribute__((ext_vector_type(2)));
+    typedef const __attribute__((address_space(1))) Pair* GlobalPtr2;
+    GlobalPtr2 pp = (GlobalPtr2)(src + xa - (long)padU * sy);
+    const int sy2 = sy / 2;
+    Pair r[N];
+    staticFor<N>([&](auto yy) {
+      constexpr int y = decltype(yy)::value;
+      r[y] = Pair{0.0f, 0.0f};
+      if ((unsigned)(y - padU) < (unsigned)h && va) r[y] = pp[(long)y * sy2];
+    });
+    staticFor<N / 2>([&](auto jj) {
+      constexpr int j = decltype(jj)::value;
+      z0[j] = c32{r[2 * j].x, r[2 * j + 1].x};
+      z1[j] = c32{r[2 * j].y, r[2 * j + 1].y};
+    });
+    return;
+  }
   GlobalPtr pa = (GlobalPtr)(src + (long)xa * sx - (long)padU * sy);
   GlobalPtr pb = pa + sx;
   float ra[N], rb[N];
