@@ -63,7 +63,8 @@ struct PlaneSet {
 };
 
 // ---- 1. planes -> S[bin][k][row] ----
-template <int N>
+// PAIRS: every plane of the set passes windowMovesAsPairs() (8-byte words per row)
+template <int N, int PAIRS>
 __global__ __launch_bounds__(kT) void forwardBinMajor(PlaneSet ps, float2* S, int Rp, int Kp,
                                                       float imSign) {
   using C = BMCfg<N>;
@@ -77,8 +78,8 @@ __global__ __launch_bounds__(kT) void forwardBinMajor(PlaneSet ps, float2* S, in
 
   c32 z0[H], z1[H];
   if (row < ps.R && k < ps.K) {
-    loadColumnsWindow<N>(ps.base + (long)row * ps.sRow + (long)k * ps.sK, ps.sy, ps.sx, ps.h, ps.w,
-                         0, 0, l, z0, z1);
+    loadColumnsWindow<N, PAIRS>(ps.base + (long)row * ps.sRow + (long)k * ps.sK, ps.sy, ps.sx,
+                                ps.h, ps.w, 0, 0, l, z0, z1);
   } else {
 #pragma unroll
     for (int j = 0; j < H; ++j) z0[j] = z1[j] = c32{0.f, 0.f};
@@ -366,8 +367,16 @@ int runPipeline(PlaneSet x, PlaneSet y, PlaneSet out, bool conjY, float scale, b
   float2* SB = SA + (size_t)bins * Kp * Ip;
   float2* SC = SB + (size_t)bins * Kp * Jp;
 
-  forwardBinMajor<N><<<dim3(Ip / SL, Kp), dim3(kT), 0, s>>>(x, SA, Ip, Kp, xSign);
-  forwardBinMajor<N><<<dim3(Jp / SL, Kp), dim3(kT), 0, s>>>(y, SB, Jp, Kp, ySign);
+  auto forward = [&](const PlaneSet& p, float2* S, int Rp, float sign) {
+    const bool pairs = windowMovesAsPairs(p.base, p.sy, p.sx, p.w, 0) && p.sRow % 2 == 0 &&
+                       p.sK % 2 == 0;
+    if (pairs)
+      forwardBinMajor<N, 1><<<dim3(Rp / SL, Kp), dim3(kT), 0, s>>>(p, S, Rp, Kp, sign);
+    else
+      forwardBinMajor<N, 0><<<dim3(Rp / SL, Kp), dim3(kT), 0, s>>>(p, S, Rp, Kp, sign);
+  };
+  forward(x, SA, Ip, xSign);
+  forward(y, SB, Jp, ySign);
   GemmArgs g;
   g.A = SA;
   g.B = SB;

@@ -33,42 +33,82 @@ __device__ __forceinline__ void ldsStore4(c32* p, c32 a, c32 b) {
 // unconditionally at an address clamped into the window and the value is zeroed
 // afterwards, so the 2N loads of a lane are all in flight together and no branch
 // separates them; the window must not be empty.  Row terms are wave-uniform.
-template <int N>
+// PAIRS = 0: one 4-byte load per sample, any strides.  PAIRS = 1: the caller
+// guarantees windowMovesAsPairs() - rows on 8-byte boundaries, even left edge and
+// width - so the lane's two columns are one 8-byte word per row, inside or outside
+// the window together.  PAIRS = 2: decided here (the test is wave-uniform).
+__host__ __device__ __forceinline__ bool windowMovesAsPairs(const float* src, long sy, long sx,
+                                                            int w, int padL) {
+  return sx == 1 && ((sy | padL | w) & 1) == 0 && (reinterpret_cast<uintptr_t>(src) & 7) == 0;
+}
+
+template <int N, int PAIRS = 2>
 __device__ __forceinline__ void loadColumnsWindow(const float* src, int sy, int sx, int h, int w,
                                                   int padL, int padU, int l, c32 (&z0)[N / 2],
                                                   c32 (&z1)[N / 2]) {
+  if constexpr (PAIRS == 2) {
+    if (windowMovesAsPairs(src, sy, sx, w, padL))
+      loadColumnsWindow<N, 1>(src, sy, sx, h, w, padL, padU, l, z0, z1);
+    else
+      loadColumnsWindow<N, 0>(src, sy, sx, h, w, padL, padU, l, z0, z1);
+    return;
+  }
   const int xa = 2 * l - padL, xb = xa + 1;
   const bool va = (unsigned)xa < (unsigned)w, vb = (unsigned)xb < (unsigned)w;
-  const float* pa = src + (long)min(max(xa, 0), w - 1) * sx;
-  const float* pb = src + (long)min(max(xb, 0), w - 1) * sx;
-  float ra[N], rb[N];
+  const int yEnd = padU + h;
   // rows in batches of 8: a batch that lies wholly below the window (the same for
   // every lane) issues no loads - a 5 x 5 filter plane costs 16 loads, not 2N
-  const int yEnd = padU + h;
-  staticFor<(N + 7) / 8>([&](auto bb) {
-    constexpr int y0 = 8 * decltype(bb)::value;
-    constexpr int y1 = y0 + 8 < N ? y0 + 8 : N;
-    if (y0 < yEnd) {
-      staticFor<y1 - y0>([&](auto yy) {
-        constexpr int y = y0 + decltype(yy)::value;
-        const long oy = (long)min(max(y - padU, 0), h - 1) * sy;
-        ra[y] = pa[oy];
-        rb[y] = pb[oy];
-      });
-    } else {
-      staticFor<y1 - y0>([&](auto yy) {
-        constexpr int y = y0 + decltype(yy)::value;
-        ra[y] = 0.0f;
-        rb[y] = 0.0f;
-      });
-    }
-  });
-  staticFor<N / 2>([&](auto jj) {
-    constexpr int j = decltype(jj)::value;
-    const bool v0 = (unsigned)(2 * j - padU) < (unsigned)h, v1 = (unsigned)(2 * j + 1 - padU) < (unsigned)h;
-    z0[j] = c32{v0 && va ? ra[2 * j] : 0.0f, v1 && va ? ra[2 * j + 1] : 0.0f};
-    z1[j] = c32{v0 && vb ? rb[2 * j] : 0.0f, v1 && vb ? rb[2 * j + 1] : 0.0f};
-  });
+  if constexpr (PAIRS == 1) {
+    const float* pp = src + min(max(xa, 0), w - 2);
+    float2 r[N];
+    staticFor<(N + 7) / 8>([&](auto bb) {
+      constexpr int y0 = 8 * decltype(bb)::value;
+      constexpr int y1 = y0 + 8 < N ? y0 + 8 : N;
+      if (y0 < yEnd) {
+        staticFor<y1 - y0>([&](auto yy) {
+          constexpr int y = y0 + decltype(yy)::value;
+          r[y] = *reinterpret_cast<const float2*>(pp + (long)min(max(y - padU, 0), h - 1) * sy);
+        });
+      } else {
+        staticFor<y1 - y0>([&](auto yy) { r[y0 + decltype(yy)::value] = float2{0.0f, 0.0f}; });
+      }
+    });
+    staticFor<N / 2>([&](auto jj) {
+      constexpr int j = decltype(jj)::value;
+      const bool v0 = va && (unsigned)(2 * j - padU) < (unsigned)h;
+      const bool v1 = va && (unsigned)(2 * j + 1 - padU) < (unsigned)h;
+      z0[j] = c32{v0 ? r[2 * j].x : 0.0f, v1 ? r[2 * j + 1].x : 0.0f};
+      z1[j] = c32{v0 ? r[2 * j].y : 0.0f, v1 ? r[2 * j + 1].y : 0.0f};
+    });
+  } else {
+    const float* pa = src + (long)min(max(xa, 0), w - 1) * sx;
+    const float* pb = src + (long)min(max(xb, 0), w - 1) * sx;
+    float ra[N], rb[N];
+    staticFor<(N + 7) / 8>([&](auto bb) {
+      constexpr int y0 = 8 * decltype(bb)::value;
+      constexpr int y1 = y0 + 8 < N ? y0 + 8 : N;
+      if (y0 < yEnd) {
+        staticFor<y1 - y0>([&](auto yy) {
+          constexpr int y = y0 + decltype(yy)::value;
+          const long oy = (long)min(max(y - padU, 0), h - 1) * sy;
+          ra[y] = pa[oy];
+          rb[y] = pb[oy];
+        });
+      } else {
+        staticFor<y1 - y0>([&](auto yy) {
+          constexpr int y = y0 + decltype(yy)::value;
+          ra[y] = 0.0f;
+          rb[y] = 0.0f;
+        });
+      }
+    });
+    staticFor<N / 2>([&](auto jj) {
+      constexpr int j = decltype(jj)::value;
+      const bool v0 = (unsigned)(2 * j - padU) < (unsigned)h, v1 = (unsigned)(2 * j + 1 - padU) < (unsigned)h;
+      z0[j] = c32{v0 && va ? ra[2 * j] : 0.0f, v1 && va ? ra[2 * j + 1] : 0.0f};
+      z1[j] = c32{v0 && vb ? rb[2 * j] : 0.0f, v1 && vb ? rb[2 * j + 1] : 0.0f};
+    });
+  }
 }
 
 // The same two columns for callers whose window geometry differs from lane to
