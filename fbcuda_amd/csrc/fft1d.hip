@@ -205,9 +205,9 @@ __global__ __launch_bounds__(k1dThreads) void fft1dInverse(Row1D a) {
 // HBM as plain 16-byte streams.
 template <int N>
 struct CfgMid {
-  static_assert(N == 64 || N == 128 || N == 256, "one, two or four lanes per row");
+  static_assert(N >= 8 && N <= 256, "one lane per row up to 64 points, then two or four");
   static constexpr int H = N / 2;
-  static constexpr int G = N / 64;          // lanes per row
+  static constexpr int G = N <= 64 ? 1 : N / 64;  // lanes per row
   static constexpr int Q = H / G;           // points per lane (32)
   static constexpr int ROWS = k1dThreads / G;
   static constexpr int RS = H + 1;          // LDS row stride (complex) = spectrum row length
@@ -569,11 +569,26 @@ int launchFft1d(bool forward, int N, float* real, int sb, int sx, float* cplx, i
   if (B <= 0) return FBFFT_SUCCESS;
   Row1D a{real, sb, sx, cplx, cb, ck, B, padL};
   const bool fast = padL == 0 && sx == 1 && sb % 2 == 0 && aligned(real, 8);
-  if ((N == 64 || N == 128 || N == 256) && padL == 0 && sx == 1 && sb == N && ck == 2 &&
-      cb == N + 2 && aligned(real, 16) && aligned(cplx, 16)) {
-    const int rowsPerGroup = k1dThreads / (N / 64);
+  if (N >= 8 && padL == 0 && sx == 1 && sb == N && ck == 2 && cb == N + 2 && aligned(real, 16) &&
+      aligned(cplx, 16)) {
+    const int rowsPerGroup = N <= 64 ? k1dThreads : k1dThreads / (N / 64);
     dim3 grid(ceilDiv(B, rowsPerGroup)), block(k1dThreads);
-    if (N == 64) {
+    if (N == 8) {
+      if (forward)
+        fft1dMidForward<8><<<grid, block, 0, s>>>(real, cplx, B);
+      else
+        fft1dMidInverse<8><<<grid, block, 0, s>>>(cplx, real, B);
+    } else if (N == 16) {
+      if (forward)
+        fft1dMidForward<16><<<grid, block, 0, s>>>(real, cplx, B);
+      else
+        fft1dMidInverse<16><<<grid, block, 0, s>>>(cplx, real, B);
+    } else if (N == 32) {
+      if (forward)
+        fft1dMidForward<32><<<grid, block, 0, s>>>(real, cplx, B);
+      else
+        fft1dMidInverse<32><<<grid, block, 0, s>>>(cplx, real, B);
+    } else if (N == 64) {
       if (forward)
         fft1dMidForward<64><<<grid, block, 0, s>>>(real, cplx, B);
       else
