@@ -75,6 +75,27 @@ __device__ __forceinline__ c32 mulRoot(c32 d) {
   }
 }
 
+// d * W / 2 with the same W: the halving is folded into the literals
+template <int M, int K, bool FWD>
+__device__ __forceinline__ c32 mulHalfRoot(c32 d) {
+  static_assert(K >= 0 && 2 * K < M, "root index");
+  if constexpr (K == 0) {
+    return c32{0.5f * d.x, 0.5f * d.y};
+  } else if constexpr (4 * K == M) {
+    return FWD ? c32{0.5f * d.y, -0.5f * d.x} : c32{-0.5f * d.y, 0.5f * d.x};
+  } else if constexpr (8 * K == M) {
+    constexpr float h = 0.5f * TableEntry<32>::c;
+    return FWD ? c32{(d.x + d.y) * h, (d.y - d.x) * h} : c32{(d.x - d.y) * h, (d.x + d.y) * h};
+  } else if constexpr (8 * K == 3 * M) {
+    constexpr float h = 0.5f * TableEntry<32>::c;
+    return FWD ? c32{(d.y - d.x) * h, -(d.x + d.y) * h} : c32{-(d.x + d.y) * h, (d.x - d.y) * h};
+  } else {
+    constexpr float c = 0.5f * TableEntry<K * 256 / M>::c;
+    constexpr float s = 0.5f * (FWD ? -TableEntry<K * 256 / M>::s : TableEntry<K * 256 / M>::s);
+    return c32{d.x * c - d.y * s, d.x * s + d.y * c};
+  }
+}
+
 // Radix-2 decimation in frequency of a[0..N): natural order in, bit-reversed
 // order out (the value with frequency index k ends up in a[bitrev(k)]).
 template <int N, bool FWD, int M = N>
@@ -119,12 +140,15 @@ __device__ __forceinline__ void realFixupForwardEmit(const c32 (&z)[H], Emit&& e
     c32 a = z[slot<H>(k)];
     c32 b = z[slot<H>(H - k)];
     // E = (a + conj b)/2, O = -i (a - conj b)/2, T = W_N^k O:
-    // F[k] = E + T, F[H-k] = conj(E - T)
-    c32 e = c32{0.5f * (a.x + b.x), 0.5f * (a.y - b.y)};
-    c32 o = c32{0.5f * (a.y + b.y), -0.5f * (a.x - b.x)};
-    c32 t = mulRoot<N, k, true>(o);
-    emit(std::integral_constant<int, k>{}, c32{e.x + t.x, e.y + t.y});
-    emit(std::integral_constant<int, H - k>{}, c32{e.x - t.x, t.y - e.y});
+    // F[k] = E + T, F[H-k] = conj(E - T).  The halvings ride on the twiddle's
+    // literals and on the final multiply-adds: 12 instructions per pair, not 16.
+    c32 e2 = c32{a.x + b.x, a.y - b.y};
+    c32 o2 = c32{a.y + b.y, b.x - a.x};
+    c32 t = mulHalfRoot<N, k, true>(o2);
+    emit(std::integral_constant<int, k>{},
+         c32{__builtin_fmaf(0.5f, e2.x, t.x), __builtin_fmaf(0.5f, e2.y, t.y)});
+    emit(std::integral_constant<int, H - k>{},
+         c32{__builtin_fmaf(0.5f, e2.x, -t.x), __builtin_fmaf(-0.5f, e2.y, t.y)});
   });
   if constexpr (H >= 2) {
     c32 a = z[slot<H>(H / 2)];
