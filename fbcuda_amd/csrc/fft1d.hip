@@ -270,11 +270,10 @@ __global__ __launch_bounds__(k1dThreads, 2) void fft1dMidForward(const float* __
     // F[k] and F[H-k] from a = Z[k], b = Z[H-k]
     auto fixBoth = [&](auto kp, c32 a, c32 bq) __attribute__((always_inline)) {
       constexpr int k = decltype(kp)::value;
-      const c32 e = c32{0.5f * (a.x + bq.x), 0.5f * (a.y - bq.y)};
-      const c32 o = c32{0.5f * (a.y + bq.y), -0.5f * (a.x - bq.x)};
-      const c32 tt = mulRoot<N, k, true>(o);
-      zrow[k] = c32{e.x + tt.x, e.y + tt.y};
-      zrow[H - k] = c32{e.x - tt.x, tt.y - e.y};
+      c32 fk, fhk;
+      realPairForward<N, k>(a, bq, fk, fhk);
+      zrow[k] = fk;
+      zrow[H - k] = fhk;
     };
     if (g == 0) {
       const c32 z0 = v[0];
@@ -318,11 +317,10 @@ __global__ __launch_bounds__(k1dThreads, 2) void fft1dMidForward(const float* __
     __syncthreads();                        // both lanes of a row have read it
     auto pairOut = [&](auto kp, c32 a, c32 bq) __attribute__((always_inline)) {
       constexpr int k = decltype(kp)::value;  // bin k pairs with H-k
-      const c32 e = c32{0.5f * (a.x + bq.x), 0.5f * (a.y - bq.y)};
-      const c32 o = c32{0.5f * (a.y + bq.y), -0.5f * (a.x - bq.x)};
-      const c32 tt = mulRoot<N, k, true>(o);
-      zrow[k] = c32{e.x + tt.x, e.y + tt.y};
-      zrow[H - k] = c32{e.x - tt.x, tt.y - e.y};
+      c32 fk, fhk;
+      realPairForward<N, k>(a, bq, fk, fhk);
+      zrow[k] = fk;
+      zrow[H - k] = fhk;
     };
     if (g == 0) {
       const c32 z0 = v[0];

@@ -186,11 +186,10 @@ __global__ __launch_bounds__(LargeCfg<N>::THREADS) void fft2dLargeForward(RealVi
     // its own half; twiddles are compile-time in both branches ----
     auto pairOut = [&](auto kp, c32 a, c32 bq) {
       constexpr int k = decltype(kp)::value;  // bin k pairs with H-k
-      c32 e = c32{0.5f * (a.x + bq.x), 0.5f * (a.y - bq.y)};
-      c32 o = c32{0.5f * (a.y + bq.y), -0.5f * (a.x - bq.x)};
-      c32 tt = mulRoot<N, k, true>(o);
-      cb[k * CS + y] = c32{e.x + tt.x, e.y + tt.y};
-      cb[(H - k) * CS + y] = c32{e.x - tt.x, tt.y - e.y};
+      c32 fk, fhk;
+      realPairForward<N, k>(a, bq, fk, fhk);
+      cb[k * CS + y] = fk;
+      cb[(H - k) * CS + y] = fhk;
     };
     if (gr == 0) {
       c32 z0 = v[0];

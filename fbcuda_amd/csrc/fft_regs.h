@@ -123,6 +123,20 @@ constexpr int slot(int k) {
   return bitrev(k, ilog2(N));
 }
 
+// F[K] and F[H-K] of the N = 2H-point real transform from a = Z[K], b = Z[H-K] of
+// the H-point transform of the even/odd packing:
+// E = (a + conj b)/2, O = -i (a - conj b)/2, T = W_N^K O, F[K] = E + T,
+// F[H-K] = conj(E - T).  The halvings ride on the twiddle's literals and on the
+// final multiply-adds: 12 instructions per pair, not 16.
+template <int N, int K>
+__device__ __forceinline__ void realPairForward(c32 a, c32 b, c32& fk, c32& fhk) {
+  const c32 e2 = c32{a.x + b.x, a.y - b.y};
+  const c32 o2 = c32{a.y + b.y, b.x - a.x};
+  const c32 t = mulHalfRoot<N, K, true>(o2);
+  fk = c32{__builtin_fmaf(0.5f, e2.x, t.x), __builtin_fmaf(0.5f, e2.y, t.y)};
+  fhk = c32{__builtin_fmaf(0.5f, e2.x, -t.x), __builtin_fmaf(-0.5f, e2.y, t.y)};
+}
+
 // Forward real-input fix-up.  z (in difFFT output order) is the H-point complex
 // FFT of z[j] = x[2j] + i*x[2j+1].  emit(k, value) is called once for every
 // k = 0..H-1 (k as an integral_constant) with F[k] of the 2H-point real
@@ -139,16 +153,10 @@ __device__ __forceinline__ void realFixupForwardEmit(const c32 (&z)[H], Emit&& e
     constexpr int k = decltype(kk)::value + 1;
     c32 a = z[slot<H>(k)];
     c32 b = z[slot<H>(H - k)];
-    // E = (a + conj b)/2, O = -i (a - conj b)/2, T = W_N^k O:
-    // F[k] = E + T, F[H-k] = conj(E - T).  The halvings ride on the twiddle's
-    // literals and on the final multiply-adds: 12 instructions per pair, not 16.
-    c32 e2 = c32{a.x + b.x, a.y - b.y};
-    c32 o2 = c32{a.y + b.y, b.x - a.x};
-    c32 t = mulHalfRoot<N, k, true>(o2);
-    emit(std::integral_constant<int, k>{},
-         c32{__builtin_fmaf(0.5f, e2.x, t.x), __builtin_fmaf(0.5f, e2.y, t.y)});
-    emit(std::integral_constant<int, H - k>{},
-         c32{__builtin_fmaf(0.5f, e2.x, -t.x), __builtin_fmaf(-0.5f, e2.y, t.y)});
+    c32 fk, fhk;
+    realPairForward<N, k>(a, b, fk, fhk);
+    emit(std::integral_constant<int, k>{}, fk);
+    emit(std::integral_constant<int, H - k>{}, fhk);
   });
   if constexpr (H >= 2) {
     c32 a = z[slot<H>(H / 2)];
