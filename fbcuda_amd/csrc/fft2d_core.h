@@ -36,7 +36,8 @@ __device__ __forceinline__ void ldsStore4(c32* p, c32 a, c32 b) {
 // PAIRS = 0: one 4-byte load per sample, any strides.  PAIRS = 1: the caller
 // guarantees windowMovesAsPairs() - rows on 8-byte boundaries, even left edge and
 // width - so the lane's two columns are one 8-byte word per row, inside or outside
-// the window together.  PAIRS = 2: decided here (the test is wave-uniform).
+// the window together.  PAIRS = 2: decided here, per lane (the planes of a wave
+// disagree only when the plane stride is odd; both paths then run under their masks).
 __host__ __device__ __forceinline__ bool windowMovesAsPairs(const float* src, long sy, long sx,
                                                             int w, int padL) {
   return sx == 1 && ((sy | padL | w) & 1) == 0 && (reinterpret_cast<uintptr_t>(src) & 7) == 0;
