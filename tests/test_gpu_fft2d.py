@@ -240,3 +240,23 @@ def test_windows_that_move_as_16_byte_words(oracle, N, h, w, padL, padU):
     _, want32 = oracle.fbfft2d(x, N, padL, padU)
     assert rel(got, want32) < TOL_FFT
     assert rel(got, oracle.dft2d_r2c(x, N, padL, padU)) < TOL_FFT
+
+
+@pytest.mark.parametrize("N", [8, 16, 32])
+def test_odd_plane_stride_mixes_the_window_load_paths(oracle, N):
+    """Even window, even row stride, odd plane stride: every other plane starts on an
+    8-byte boundary, so the planes of one wave take different load paths."""
+    B, h, w = 11, N // 2, N // 2 - 2
+    x = synth.normal((B, h, w), seed=5 * N).numpy()
+    flat = torch.zeros(B * (h * w + 1) + 8, device=dev())
+    real = flat.as_strided((B, h, w), (h * w + 1, w, 1))
+    real.copy_(torch.from_numpy(x))
+    spec = torch.full((B, N // 2 + 1, N, 2), float("nan"), device=dev())
+    assert F.fbfft2D(real, spec, 2, 1) == F.Success
+    torch.cuda.synchronize()
+    _, want = oracle.fbfft2d(x, N, 2, 1)
+    assert rel(spec.cpu().numpy(), want) < TOL_FFT
+    back = torch.zeros_like(flat).as_strided((B, h, w), (h * w + 1, w, 1))
+    assert F.fbifft2D(spec, back, 2, 1) == F.Success
+    torch.cuda.synchronize()
+    assert rel(back.cpu().numpy(), N * N * x.astype(np.float64)) < TOL_FFT
