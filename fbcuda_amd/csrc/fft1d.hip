@@ -189,10 +189,10 @@ __global__ __launch_bounds__(k1dThreads) void fft1dInverse(Row1D a) {
   }
 }
 
-// ---- N = 64, 128 and 256 with contiguous, 16-byte aligned operands ----
+// ---- N = 8 ... 256 with contiguous, 16-byte aligned operands ----
 //
 // Same staging as above, but the real-input fix-up never makes a pass of its own
-// through LDS: with one lane per row (N = 64) the whole half-length transform is in
+// through LDS: with one lane per row (N <= 64) the whole half-length transform is in
 // the lane's registers, and with two lanes per row (N = 128) the split is chosen so
 // that the fix-up pairs (k, N/2 - k) stay inside one lane - the forward transform
 // splits its outputs by parity, the inverse its inputs (E = IFFT(z even),
