@@ -154,6 +154,10 @@ __global__ __launch_bounds__(64) void fft2dSmallForward(RealView real, CplxView 
   }
 }
 
+__device__ __forceinline__ bool aligned16(const void* p) {
+  return (reinterpret_cast<uintptr_t>(p) & 15) == 0;
+}
+
 template <int N, bool FAST_REAL, bool FAST_CPLX, int GPW>
 __global__ __launch_bounds__(64) void fft2dSmallInverse(CplxView cplx, RealView real, int padL,
                                                         int padU) {
@@ -227,6 +231,32 @@ __global__ __launch_bounds__(64) void fft2dSmallInverse(CplxView cplx, RealView 
     c32 z0[H], z1[H];
     columnPassInverse<N>(plane, l, z0, z1);
     const int b = b0 + pl;
+    if constexpr (FAST_REAL && N <= 16) {
+      // Rows of 32 or 64 bytes: stored from the column layout, a wave instruction
+      // would touch 16 or 8 cache lines with a fraction of each.  When the planes
+      // of the group are contiguous in memory they go back through LDS instead and
+      // leave as one stream of 16-byte stores.
+      if (real.sy == N && real.sb == N * N && aligned16(real.data)) {
+        __syncthreads();  // the spectra have been consumed
+        float* stage = reinterpret_cast<float*>(lds);
+        float* mine = stage + pl * N * N + 2 * l;
+        staticFor<H>([&](auto jj) {
+          constexpr int j = decltype(jj)::value;
+          c32 a = z0[slot<H>(j)], c = z1[slot<H>(j)];
+          *reinterpret_cast<float2*>(mine + (2 * j) * N) = float2{a.x, c.x};
+          *reinterpret_cast<float2*>(mine + (2 * j + 1) * N) = float2{a.y, c.y};
+        });
+        __syncthreads();
+        const int valid = min(P, B - b0) * (N * N / 4);  // float4 of the group's planes
+        float4* dst = reinterpret_cast<float4*>(real.data + (size_t)b0 * (N * N));
+        staticFor<P * N * N / 4 / 64>([&](auto ii) {
+          constexpr int i = decltype(ii)::value;
+          const int q = lane + 64 * i;
+          if (q < valid) dst[q] = reinterpret_cast<const float4*>(stage)[q];
+        });
+        return;
+      }
+    }
     if (b < B) {
       if constexpr (FAST_REAL) {
         float2* dst = reinterpret_cast<float2*>(real.data + (size_t)b * real.sb) + l;
