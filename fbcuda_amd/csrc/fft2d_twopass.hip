@@ -9,6 +9,8 @@
 // transform's points are gathered and where its results go, so one kernel serves
 // them: a 256-lane workgroup stages 256/G transforms in LDS (G = N/32 lanes per
 // transform), runs the radix-G split + 32-point in-register FFT and scatters.
+// The transposed reads of the second passes are coalesced by running the lanes
+// along the transform index (consecutive transforms are adjacent in memory).
 #include "common.h"
 #include "fft_lds.h"
 #include "fft_regs.h"
@@ -51,32 +53,56 @@ __global__ __launch_bounds__(kTP) void twoPassKernel(TwoPassArgs a, int total) {
     return c32{v.x, -v.y};
   };
 
-  for (int idx = t; idx < ROWS * N; idx += kTP) {
-    const int qi = idx / N, j = idx % N;
-    const int q = q0 + qi;
-    c32 v = c32{0.f, 0.f};
-    if (q < total) {
+  // Gather ROWS transforms of N points.  Lanes run along whichever index is
+  // contiguous in the source: the point index j for modes 0 and 2, the transform
+  // index for modes 1 and 3 (the transposed reads of the second passes).  Loads go
+  // out in batches of 16 at clamped coordinates with no branch between them; what
+  // lies outside the window or beyond the last transform is zeroed or ignored later.
+  constexpr bool ALONG_Q = MODE == 1 || MODE == 3;
+  constexpr int ITER = ROWS * N / kTP, BATCH = 16;
+  static_assert(ITER % BATCH == 0, "whole batches");
+#pragma unroll
+  for (int i0 = 0; i0 < ITER; i0 += BATCH) {
+    float vx[BATCH], vy[BATCH];
+#pragma unroll
+    for (int u = 0; u < BATCH; ++u) {
+      const int idx = t + kTP * (i0 + u);
+      const int qi = ALONG_Q ? idx % ROWS : idx / N, j = ALONG_Q ? idx / ROWS : idx % N;
+      const int q = min(q0 + qi, total - 1);
+      c32 v = c32{0.f, 0.f};
       if (MODE == 0) {
         const int b = q / N, y = q % N;
-        if (inWindow(y, j, a.padU, a.padL, a.h, a.w))
-          v.x = a.src[(long)b * a.s0 + (long)(y - a.padU) * a.s1 + (long)(j - a.padL) * a.s2];
+        const int ys = min(max(y - a.padU, 0), a.h - 1), xs = min(max(j - a.padL, 0), a.w - 1);
+        v.x = a.src[(long)b * a.s0 + (long)ys * a.s1 + (long)xs * a.s2];
       } else if (MODE == 1) {
         const int b = q / nc, kx = q % nc;
         v = cplxAt(a.src + (long)b * a.s0 + (long)j * a.s1 + (long)kx * a.s2);
       } else if (MODE == 2) {
         const int b = q / N, row = q % N;
         v = expand(b, row, j);
+        const c32 w = expand(min(b + half, a.B - 1), row, j);
         if (b + half < a.B) {
-          c32 u = expand(b + half, row, j);
-          v.x -= u.y;  // + i * u
-          v.y += u.x;
+          v.x -= w.y;  // + i * w
+          v.y += w.x;
         }
       } else {
         const int b = q / N, x = q % N;
         v = cplxAt(a.src + (long)b * a.s0 + (long)j * a.s1 + (long)x * a.s2);
       }
+      vx[u] = v.x;
+      vy[u] = v.y;
     }
-    lds[qi * RS + j] = v;
+#pragma unroll
+    for (int u = 0; u < BATCH; ++u) {
+      const int idx = t + kTP * (i0 + u);
+      const int qi = ALONG_Q ? idx % ROWS : idx / N, j = ALONG_Q ? idx / ROWS : idx % N;
+      c32 v = c32{vx[u], vy[u]};
+      if (MODE == 0) {
+        const int y = min(q0 + qi, total - 1) % N;
+        if (!inWindow(y, j, a.padU, a.padL, a.h, a.w)) v.x = 0.0f;
+      }
+      lds[qi * RS + j] = v;
+    }
   }
   __syncthreads();
 
@@ -91,15 +117,18 @@ __global__ __launch_bounds__(kTP) void twoPassKernel(TwoPassArgs a, int total) {
   });
   __syncthreads();
 
-  for (int idx = t; idx < ROWS * N; idx += kTP) {
-    const int qi = idx / N, k = idx % N;
+  // results leave along their contiguous index k; the first forward pass keeps
+  // N/2+1 of its N bins
+  constexpr int KEEP = MODE == 0 ? nc : N;
+#pragma unroll 4
+  for (int idx = t; idx < ROWS * KEEP; idx += kTP) {
+    const int qi = idx / KEEP, k = idx % KEEP;
     const int q = q0 + qi;
     if (q >= total) break;
     const c32 r = lds[qi * RS + k];
     if (MODE == 0) {
       const int b = q / N, y = q % N;
-      if (k < nc)
-        *reinterpret_cast<float2*>(a.dst + (long)b * a.d0 + (long)y * a.d1 + (long)k * a.d2) = r;
+      *reinterpret_cast<float2*>(a.dst + (long)b * a.d0 + (long)y * a.d1 + (long)k * a.d2) = r;
     } else if (MODE == 1) {
       const int b = q / nc, kx = q % nc;
       *reinterpret_cast<float2*>(a.dst + (long)b * a.d0 + (long)kx * a.d1 + (long)k * a.d2) = r;
