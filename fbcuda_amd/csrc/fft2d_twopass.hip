@@ -61,6 +61,36 @@ __global__ __launch_bounds__(kTP) void twoPassKernel(TwoPassArgs a, int total) {
   constexpr bool ALONG_Q = MODE == 1 || MODE == 3;
   constexpr int ITER = ROWS * N / kTP, BATCH = 16;
   static_assert(ITER % BATCH == 0, "whole batches");
+  // real rows on 16-byte boundaries, window edge and width multiples of 4: 16-byte loads
+  const bool vec = MODE == 0 && a.s2 == 1 && ((a.s1 | a.s0 | a.padL | a.w) & 3) == 0 &&
+                   (reinterpret_cast<uintptr_t>(a.src) & 15) == 0;
+  if (vec) {
+    constexpr int I4 = ITER / 4;  // 8 float4 per lane
+    float v4[4 * I4];
+#pragma unroll
+    for (int u = 0; u < I4; ++u) {
+      const int idx = t + kTP * u;
+      const int qi = idx / (N / 4), j4 = idx % (N / 4);
+      const int q = min(q0 + qi, total - 1);
+      const int b = q / N, y = q % N;
+      const int ys = min(max(y - a.padU, 0), a.h - 1), xs = min(max(4 * j4 - a.padL, 0), a.w - 4);
+      const float4 w = *reinterpret_cast<const float4*>(a.src + (long)b * a.s0 + (long)ys * a.s1 + xs);
+      v4[4 * u] = w.x;
+      v4[4 * u + 1] = w.y;
+      v4[4 * u + 2] = w.z;
+      v4[4 * u + 3] = w.w;
+    }
+#pragma unroll
+    for (int u = 0; u < I4; ++u) {
+      const int idx = t + kTP * u;
+      const int qi = idx / (N / 4), j4 = idx % (N / 4);
+      const int y = min(q0 + qi, total - 1) % N;
+      const bool in = inWindow(y, 4 * j4, a.padU, a.padL, a.h, a.w);
+      c32* d = lds + qi * RS + 4 * j4;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) d[e] = c32{in ? v4[4 * u + e] : 0.0f, 0.0f};
+    }
+  } else
 #pragma unroll
   for (int i0 = 0; i0 < ITER; i0 += BATCH) {
     float vx[BATCH], vy[BATCH];

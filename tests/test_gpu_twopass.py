@@ -13,10 +13,12 @@ pytestmark = pytest.mark.gpu
 
 @pytest.mark.parametrize("N", [64, 128])
 @pytest.mark.parametrize("B", [1, 4, 5])
-@pytest.mark.parametrize("case", ["full", "padded"])
+@pytest.mark.parametrize("case", ["full", "padded", "aligned", "aligned_narrow"])
 def test_two_call_forward_and_inverse(oracle, N, B, case):
     d = dev()
-    h, w, padL, padU = (N, N, 0, 0) if case == "full" else (N - 9, N - 6, 4, 3)
+    # "aligned*": width and left edge multiples of 4 (16-byte loads of the first pass)
+    h, w, padL, padU = {"full": (N, N, 0, 0), "padded": (N - 9, N - 6, 4, 3),
+                        "aligned": (N - 9, N - 8, 4, 3), "aligned_narrow": (7, 12, 8, 0)}[case]
     x = synth.normal((B, h, w), seed=N + B).numpy()
     xd = torch.from_numpy(x).to(d)
     nc = N // 2 + 1
