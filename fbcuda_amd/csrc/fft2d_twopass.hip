@@ -46,11 +46,12 @@ __global__ __launch_bounds__(kTP) void twoPassKernel(TwoPassArgs a, int total) {
 
   auto cplxAt = [](const float* p) { return *reinterpret_cast<const float2*>(p); };
   // Hermitian expansion of the half spectrum [N/2+1][N] (fbfft/FBIFFT2D-inl.cuh:61-97)
+  // (one load at a selected address, so that the loads of a batch stay free of branches)
   auto expand = [&](int b, int row, int col) {
-    const float* p = a.src + (long)b * a.s0;
-    if (row < nc) return cplxAt(p + (long)row * a.s1 + (long)col * a.s2);
-    c32 v = cplxAt(p + (long)(N - row) * a.s1 + (long)((N - col) % N) * a.s2);
-    return c32{v.x, -v.y};
+    const bool stored = row < nc;
+    const int r = stored ? row : N - row, c = stored ? col : (N - col) % N;
+    c32 v = cplxAt(a.src + (long)b * a.s0 + (long)r * a.s1 + (long)c * a.s2);
+    return c32{v.x, stored ? v.y : -v.y};
   };
 
   // Gather ROWS transforms of N points.  Lanes run along whichever index is
