@@ -261,8 +261,11 @@ def run_only(name, steps, warmup, F, synth, torch, dev):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=20)
+    # defaults: 3000 launches of 23 us.  Launched over and over on the same 132 MB the
+    # kernel keeps getting faster for about a thousand launches (24 -> 22 us) while the
+    # last-level cache settles; the default warm-up runs past that.
+    ap.add_argument("--steps", type=int, default=2000)
+    ap.add_argument("--warmup", type=int, default=1000)
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the informative extra configs")
     ap.add_argument("--only", default=None,
