@@ -130,7 +130,7 @@ def conv_extras(F, synth, torch, dev, extra):
                                 stream)
         if rc != 0:
             raise RuntimeError(F.error_string(rc))
-    _, t = timed(conv, 50, 5, torch)
+    _, t = timed(conv, 200, 200, torch)
     extra["fft_conv_configs3_ms_per_iter"] = round(t * 1e3, 4)
     extra["fft_conv_configs3_direct_equiv_TFLOPs"] = round(41.6e9 / t / 1e12, 1)
     extra["fft_conv_configs3_fp32_peak_direct_ms"] = round(41.6e9 / 157.3e12 * 1e3, 4)
@@ -151,16 +151,16 @@ def conv_extras(F, synth, torch, dev, extra):
         if L.fbfft_conv_accgrad(ctypes.byref(vx), ctypes.byref(vg), ctypes.byref(vgw), 32,
                                 ctypes.c_float(1.0), 0, wsp2, wsb2, stream) != 0:
             raise RuntimeError("fbfft_conv_accgrad failed")
-    _, t = timed(bprop, 50, 5, torch)
+    _, t = timed(bprop, 200, 200, torch)
     extra["fft_conv_configs3_bprop_ms_per_iter"] = round(t * 1e3, 4)
-    _, t = timed(accgrad, 50, 5, torch)
+    _, t = timed(accgrad, 200, 200, torch)
     extra["fft_conv_configs3_accgrad_ms_per_iter"] = round(t * 1e3, 4)
     del g, gi, gw, ws2
     A = synth.normal((128, 64, 17, 32, 2), seed=30, device=dev)
     Bm = synth.normal((192, 64, 17, 32, 2), seed=31, device=dev)
     C = torch.empty((128, 192, 17, 32, 2), device=dev)
     mm = prepared("fbfft_transpose_mm", F, A, Bm, C, 0, 1, 0, ctypes.c_float(1.0 / 1024))
-    _, t = timed(mm, 50, 5, torch)
+    _, t = timed(mm, 200, 200, torch)
     extra["transposeMM_configs3_us"] = round(t * 1e6, 1)
     extra["transposeMM_configs3_TFLOPs"] = round(6.845e9 / t / 1e12, 1)
     extra["transposeMM_configs3_frac_of_fp32_mfma_peak"] = round(6.845e9 / t / 157.3e12, 4)
@@ -176,7 +176,7 @@ def conv_extras(F, synth, torch, dev, extra):
         if L.fbfft_conv_fprop(ctypes.byref(v6[0]), ctypes.byref(v6[1]), ctypes.byref(v6[2]), 64,
                               ctypes.c_void_p(ws6.data_ptr()), ws6.numel(), stream) != 0:
             raise RuntimeError("fbfft_conv_fprop (64) failed")
-    _, t = timed(conv64, 50, 5, torch)
+    _, t = timed(conv64, 200, 200, torch)
     flop64 = 2.0 * 32 * 64 * 56 * 56 * 32 * 25
     extra["fft_conv_64pt_32x32x60x60_k5_f64_ms_per_iter"] = round(t * 1e3, 4)
     extra["fft_conv_64pt_direct_equiv_TFLOPs"] = round(flop64 / t / 1e12, 1)
@@ -194,7 +194,7 @@ def conv_extras(F, synth, torch, dev, extra):
                                    ctypes.c_float(1.0), 16, n, stream)
         if rc != 1:
             raise RuntimeError("fbfft_iterated_conv returned %d" % rc)
-    _, t = timed(tiled, 10, 2, torch)
+    _, t = timed(tiled, 30, 20, torch)
     extra["iterated_conv_configs4_ms_per_iter"] = round(t * 1e3, 4)
     extra["iterated_conv_configs4_direct_equiv_TFLOPs"] = round(163.3e9 / t / 1e12, 1)
     # the other two passes over the same descriptors (o4 as gradOutput)
@@ -205,7 +205,7 @@ def conv_extras(F, synth, torch, dev, extra):
                                        ctypes.c_float(1.0), 16, n, stream)
             if rc != 1:
                 raise RuntimeError("fbfft_iterated_conv returned %d" % rc)
-        _, t = timed(other, 5, 1, torch)
+        _, t = timed(other, 30, 20, torch)
         extra["iterated_conv_configs4_%s_ms_per_iter" % key] = round(t * 1e3, 4)
 
 
