@@ -77,7 +77,9 @@ __global__ __launch_bounds__(64) void fft2dSmallForward(RealView real, CplxView 
   };
 
   // copy out: (H+1) x N complex per plane, rows 0 and H unpacked from packed row 0
-  auto copyOut = [&](int b0) __attribute__((always_inline)) {
+  // (FULL: every plane of the group exists, the common case - no per-store test)
+  auto copyOutImpl = [&](int b0, auto fullTag) __attribute__((always_inline)) {
+    constexpr bool FULL = decltype(fullTag)::value;
     staticFor<C::ITERS>([&](auto tt) {
       constexpr int t = decltype(tt)::value;
       // One iteration stores 64 / (N/2) consecutive spectral rows.  When none of
@@ -89,7 +91,7 @@ __global__ __launch_bounds__(64) void fft2dSmallForward(RealView real, CplxView 
         const int g = lane / (N / 2), xq = lane % (N / 2);
         const float4 v = ldsLoad4(lds + pp0 * PS + (r0 + g) * RS + 2 * xq);
         const int bo = b0 + pp0;
-        if (bo < B) {
+        if (FULL || bo < B) {
           if constexpr (FAST_CPLX) {
             reinterpret_cast<float4*>(cplx.data + (size_t)bo * cplx.sb)[(r0 + g) * (N / 2) + xq] = v;
           } else {
@@ -122,7 +124,7 @@ __global__ __launch_bounds__(64) void fft2dSmallForward(RealView real, CplxView 
         v = ldsLoad4(base + r * RS + kx);
       }
       const int bo = b0 + pp;
-      if (bo < B) {
+      if (FULL || bo < B) {
         if constexpr (FAST_CPLX) {
           reinterpret_cast<float4*>(cplx.data + (size_t)bo * cplx.sb)[rem] = v;
         } else {
@@ -132,6 +134,12 @@ __global__ __launch_bounds__(64) void fft2dSmallForward(RealView real, CplxView 
         }
       }
     });
+  };
+  auto copyOut = [&](int b0) __attribute__((always_inline)) {
+    if (b0 + P <= B)
+      copyOutImpl(b0, std::true_type{});
+    else
+      copyOutImpl(b0, std::false_type{});
   };
 
   const int g0 = blockIdx.x * GPW * P;
