@@ -104,7 +104,31 @@ inline fbfft_tensor describe(const DeviceTensor<Complex, Dim>& t) {
 
 }  // namespace fbfft_amd_detail
 
+// The padding predicate of MemoryAccess.cuh:11-54: sample (y, x) of the padded
+// plane lies inside the tensor's window placed at (padU, padL); one unsigned
+// compare per axis tests both bounds.
+inline bool inBounds(int x, int padL, const DeviceTensor<float, 2>& t) {
+  return (unsigned)(x - padL) < (unsigned)t.getSize(1);
+}
+inline bool inBounds(int y, int x, int padU, int padL, const DeviceTensor<float, 3>& t) {
+  return (unsigned)(y - padU) < (unsigned)t.getSize(1) &&
+         (unsigned)(x - padL) < (unsigned)t.getSize(2);
+}
+inline bool inBounds(int y, int x, int padU, int padL, const DeviceTensor<float, 4>& t) {
+  return (unsigned)(y - padU) < (unsigned)t.getSize(2) &&
+         (unsigned)(x - padL) < (unsigned)t.getSize(3);
+}
+inline bool inBounds(int x, const DeviceTensor<float, 2>& t) {
+  return (unsigned)x < (unsigned)t.getSize(1);
+}
+
 namespace fbfft {
+
+// number of stored bins of a Hermitian half spectrum (FBFFTCommon.cuh:19-22)
+template <typename T>
+inline T numHermitian(T commonCols) {
+  return commonCols / 2 + 1;
+}
 
 class FBFFTParameters {
  public:

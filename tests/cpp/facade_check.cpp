@@ -13,6 +13,8 @@
 #include "cuda/fbfft/FBFFT.cuh"
 #include "cuda/MM.cuh"
 #include "cuda/fbfft/FFTIteratedConvolution.cuh"
+#include "cuda/fbfft/FBFFTCommon.cuh"
+#include "cuda/MemoryAccess.cuh"
 
 using namespace facebook::cuda;
 using facebook::cuda::fbfft::FBFFTParameters;
@@ -164,6 +166,15 @@ double convLayerError() {
 }  // namespace
 
 int main() {
+  {  // host helpers of the reference's headers
+    using namespace facebook::cuda;
+    if (fbfft::numHermitian(32) != 17 || fbfft::numHermitian(2) != 2) return 1;
+    int sz3[3] = {4, 5, 7};
+    DeviceTensor<float, 3> t3(nullptr, sz3);
+    if (!inBounds(2, 3, 2, 3, t3) || !inBounds(6, 9, 2, 3, t3) || inBounds(7, 3, 2, 3, t3) ||
+        inBounds(1, 3, 2, 3, t3) || inBounds(2, 10, 2, 3, t3))
+      return 1;
+  }
   const int B = 3, N = 32, nc = N / 2 + 1;
   std::vector<float> x((size_t)B * N * N);
   unsigned s = 12345u;
