@@ -11,7 +11,7 @@ without the built library raises.
 import ctypes
 import os
 
-from .params import FBFFTParameters  # noqa: F401
+from .params import FBFFTParameters, numHermitian  # noqa: F401
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "csrc", "libfbfft_amd.so")

@@ -54,3 +54,8 @@ class FBFFTParameters:
 
     def padUp(self):
         return self._pad_up
+
+
+def numHermitian(commonCols):
+    """Stored bins of a Hermitian half spectrum (fbfft/FBFFTCommon.cuh:19-22)."""
+    return commonCols // 2 + 1

@@ -63,6 +63,7 @@ def test_parameters_mirror():
     assert q is p and p.inverseFFT() and p.normalizeFFT() and (p.padLeft(), p.padUp()) == (3, 4)
     assert p.forward().forwardFFT()
     assert (p.Success, p.UnsupportedSize, p.UnsupportedDimension, p.CudaError) == (0, 1, 2, 3)
+    assert [F.numHermitian(n) for n in (2, 8, 32, 256)] == [2, 5, 17, 129]
 
 
 def test_cpu_tensors_are_rejected():
