@@ -48,7 +48,7 @@ EXPORTS = (
     "fbfft_r2c_1d", "fbfft_c2r_1d", "fbfft_r2c_2d", "fbfft_c2c_2d_pass2", "fbfft_c2r_2d",
     "fbfft_c2c_2d_inverse_pass1", "fbfft_transpose_mm", "fbfft_iterated_conv", "fbfft_make_tiles",
     "fbfft_conv_workspace", "fbfft_conv_fprop_workspace", "fbfft_conv_fprop", "fbfft_conv_bprop",
-    "fbfft_conv_accgrad", "fbfft_error_string",
+    "fbfft_conv_accgrad", "fbfft_conv_fprop_static", "fbfft_error_string",
     "fbfft_twiddle_table",
 )
 
@@ -85,6 +85,7 @@ def lib():
         L.fbfft_conv_bprop.argtypes = [tp, tp, tp, ctypes.c_int, vp, ctypes.c_size_t, vp]
         L.fbfft_conv_accgrad.argtypes = [tp, tp, tp, ctypes.c_int, ctypes.c_float, ctypes.c_int, vp,
                                          ctypes.c_size_t, vp]
+        L.fbfft_conv_fprop_static.argtypes = [tp, tp, tp, ctypes.c_int, vp]
         L.fbfft_error_string.argtypes = [ctypes.c_int]
         L.fbfft_error_string.restype = ctypes.c_char_p
         L.fbfft_twiddle_table.argtypes = [ctypes.POINTER(ctypes.c_float)]
@@ -236,6 +237,18 @@ def conv_fprop(input, weight, output, fftSize, workspace, stream=None):
     return lib().fbfft_conv_fprop(view(input), view(weight), view(output), fftSize,
                                   ctypes.c_void_p(workspace.data_ptr()),
                                   workspace.numel() * workspace.element_size(), _stream(stream))
+
+
+STATIC_SCRATCH_BYTES = 32 << 20
+
+
+def conv_fprop_static(input, weight, output, fftSize, stream=None):
+    """conv_fprop through the library's own fixed scratch array (fbfft_conv_fprop_static):
+    no workspace argument, no allocation; layers needing more than STATIC_SCRATCH_BYTES of
+    workspace return UnsupportedSize."""
+    _on_gpu(input, weight, output)
+    return lib().fbfft_conv_fprop_static(view(input), view(weight), view(output), fftSize,
+                                         _stream(stream))
 
 
 def conv_workspace(pass_, batch, cin, cout, fftSize):

@@ -186,6 +186,19 @@ int fbfft_conv_accgrad(const fbfft_tensor* input, const fbfft_tensor* gradOutput
                        int accumulate, void* workspace, size_t workspaceBytes,
                        fbfft_stream_t stream);
 
+/* fbfft_conv_fprop without a workspace argument and without any allocation.  It
+ * has no counterpart in the reference; it is for callers that cannot allocate
+ * device memory: code under HIP graph capture, tight serving loops, harnesses
+ * that forbid hipMalloc.  The spectra pass through a fixed array of
+ * FBFFT_STATIC_SCRATCH_BYTES in the library's device image (each GPU the library
+ * runs on holds its own copy until the process ends).  Layers whose
+ * fbfft_conv_workspace(0, ...) exceeds that size return UnsupportedSize.  All
+ * calls on one GPU share that GPU's array: calls on one stream are ordered, calls
+ * that overlap in time on one GPU race.  Results are those of fbfft_conv_fprop. */
+#define FBFFT_STATIC_SCRATCH_BYTES (32u << 20)
+int fbfft_conv_fprop_static(const fbfft_tensor* input, const fbfft_tensor* weight,
+                            const fbfft_tensor* output, int fftSize, fbfft_stream_t stream);
+
 /* Human-readable name of an fbfft_error. */
 const char* fbfft_error_string(int code);
 
