@@ -197,12 +197,14 @@ def conv_extras(F, synth, torch, dev, extra):
     _, t = timed(tiled, 30, 20, torch)
     extra["iterated_conv_configs4_ms_per_iter"] = round(t * 1e3, 4)
     extra["iterated_conv_configs4_direct_equiv_TFLOPs"] = round(163.3e9 / t / 1e12, 1)
-    # the other two passes over the same descriptors (o4 as gradOutput)
-    for pass_, key in ((1, "bprop"), (2, "accgrad")):
+    # the other two passes (o4 as gradOutput): accGradParameters on the same descriptors,
+    # updateGradInput on its own grid of disjoint gradInput windows
+    bins, bouts, nbp = F.make_tile_grid(x4, o4, 9, 9, 32, F.FFT_UpdateGradInput)
+    for pass_, key, ti, to, nt in ((1, "bprop", bins, bouts, nbp), (2, "accgrad", ins, outs, n)):
         def other():
-            rc = L.fbfft_iterated_conv(32, ctypes.c_void_p(ins.data_ptr()),
-                                       ctypes.c_void_p(outs.data_ptr()), ctypes.byref(vw4), pass_,
-                                       ctypes.c_float(1.0), 16, n, stream)
+            rc = L.fbfft_iterated_conv(32, ctypes.c_void_p(ti.data_ptr()),
+                                       ctypes.c_void_p(to.data_ptr()), ctypes.byref(vw4), pass_,
+                                       ctypes.c_float(1.0), 16, nt, stream)
             if rc != 1:
                 raise RuntimeError("fbfft_iterated_conv returned %d" % rc)
         _, t = timed(other, 30, 20, torch)

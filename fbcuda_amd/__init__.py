@@ -47,6 +47,7 @@ _lib = None
 EXPORTS = (
     "fbfft_r2c_1d", "fbfft_c2r_1d", "fbfft_r2c_2d", "fbfft_c2c_2d_pass2", "fbfft_c2r_2d",
     "fbfft_c2c_2d_inverse_pass1", "fbfft_transpose_mm", "fbfft_iterated_conv", "fbfft_make_tiles",
+    "fbfft_make_tiles_for_pass",
     "fbfft_conv_workspace", "fbfft_conv_fprop_workspace", "fbfft_conv_fprop", "fbfft_conv_bprop",
     "fbfft_conv_accgrad", "fbfft_conv_fprop_static", "fbfft_error_string",
     "fbfft_twiddle_table",
@@ -77,6 +78,9 @@ def lib():
         L.fbfft_make_tiles.argtypes = [tp, tp, ctypes.c_int, ctypes.c_int, ctypes.c_int, vp, vp,
                                        ctypes.c_size_t]
         L.fbfft_make_tiles.restype = ctypes.c_size_t
+        L.fbfft_make_tiles_for_pass.argtypes = [ctypes.c_int, tp, tp, ctypes.c_int, ctypes.c_int,
+                                                ctypes.c_int, vp, vp, ctypes.c_size_t]
+        L.fbfft_make_tiles_for_pass.restype = ctypes.c_size_t
         L.fbfft_conv_fprop_workspace.argtypes = [ctypes.c_int] * 4
         L.fbfft_conv_fprop_workspace.restype = ctypes.c_size_t
         L.fbfft_conv_fprop.argtypes = [tp, tp, tp, ctypes.c_int, vp, ctypes.c_size_t, vp]
@@ -109,6 +113,9 @@ def view(t):
     d.data = t.data_ptr()
     d.dim = t.dim()
     for i in range(t.dim()):
+        # the descriptor holds 32-bit ints like DeviceTensor (DeviceTensor.cuh:241-245)
+        if not (0 <= t.size(i) < 2 ** 31 and -2 ** 31 <= t.stride(i) < 2 ** 31):
+            raise ValueError("size or stride of dimension %d does not fit a 32-bit int" % i)
         d.size[i] = t.size(i)
         d.stride[i] = t.stride(i)
     return d
@@ -195,18 +202,21 @@ def make_tiles(t, windows):
     return host.to(t.device), len(windows)
 
 
-def make_tile_grid(input, output, kH, kW, fftSize):
-    """The overlap tiling of a whole layer (fbfft_make_tiles): device descriptor
-    arrays (ins, outs) for `input` [B][Cin][H][W] and `output` [B][Cout][H-kH+1][W-kW+1],
-    and the tile count.  Raises on unsupported arguments."""
+def make_tile_grid(input, output, kH, kW, fftSize, pass_=FFT_UpdateOutput):
+    """The tiling of a whole layer for one pass (fbfft_make_tiles_for_pass): device
+    descriptor arrays (ins, outs) for `input` [B][Cin][H][W] and `output`
+    [B][Cout][H-kH+1][W-kW+1], and the tile count.  FFT_UpdateGradInput has its own
+    grid (disjoint gradInput windows); the other two passes share one.  Raises on
+    unsupported arguments."""
     import torch
     vi, vo = view(input), view(output)
-    n = lib().fbfft_make_tiles(vi, vo, kH, kW, fftSize, None, None, 0)
+    n = lib().fbfft_make_tiles_for_pass(int(pass_), vi, vo, kH, kW, fftSize, None, None, 0)
     if n == 0:
-        raise ValueError("fbfft_make_tiles: unsupported arguments")
+        raise ValueError("fbfft_make_tiles_for_pass: unsupported arguments")
     a, b = (Tile * n)(), (Tile * n)()
-    got = lib().fbfft_make_tiles(vi, vo, kH, kW, fftSize, ctypes.cast(a, ctypes.c_void_p),
-                                 ctypes.cast(b, ctypes.c_void_p), n)
+    got = lib().fbfft_make_tiles_for_pass(int(pass_), vi, vo, kH, kW, fftSize,
+                                          ctypes.cast(a, ctypes.c_void_p),
+                                          ctypes.cast(b, ctypes.c_void_p), n)
     assert got == n
     up = lambda arr: torch.frombuffer(bytearray(bytes(arr)), dtype=torch.uint8).to(input.device)
     return up(a), up(b), n

@@ -63,6 +63,24 @@ int collapsedBins(const fbfft_tensor* t) {
   return (int)xy;
 }
 
+// cplx[b][r][c] = 0 through the view's strides: the transform of an empty real
+// window (all padding) is all zeros
+__global__ void zeroSpectrum(CplxView v) {
+  const long per = (long)v.rows * v.cols, total = per * v.B;
+  for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total;
+       i += (long)gridDim.x * blockDim.x) {
+    const long b = i / per, rc = i % per;
+    float* p = v.data + b * v.sb + (rc / v.cols) * v.sr + (rc % v.cols) * v.sc;
+    *reinterpret_cast<float2*>(p) = float2{0.0f, 0.0f};
+  }
+}
+
+int launchZeroSpectrum(const CplxView& v, hipStream_t s) {
+  const long total = (long)v.B * v.rows * v.cols;
+  zeroSpectrum<<<dim3((unsigned)std::min<long>((total + 255) / 256, 8192)), 256, 0, s>>>(v);
+  return launchStatus();
+}
+
 }  // namespace
 
 extern "C" {
@@ -123,7 +141,9 @@ int fbfft_r2c_2d(const fbfft_tensor* real, const fbfft_tensor* cplx, int padL, i
   if (real->size[1] > N || real->size[2] > N || padL < 0 || padU < 0)
     return FBFFT_UNSUPPORTED_SIZE;
   if (!okCplx(cplx)) return FBFFT_UNSUPPORTED_DIMENSION;
-  if (empty(real) || empty(cplx)) return FBFFT_SUCCESS;
+  if (empty(cplx)) return FBFFT_SUCCESS;
+  // B > 0 planes with an empty real window: every sample is padding
+  if (empty(real)) return launchZeroSpectrum(cplxView4(cplx), stream);
   if (N < 8) return launchFft2dTinyForward(N, realView3(real), cplxView4(cplx), padL, padU, stream);
   if (N <= 32) return launchFft2dSmallForward(N, realView3(real), cplxView4(cplx), padL, padU, stream);
   if (!scratchForm)
@@ -285,10 +305,12 @@ extern "C" int fbfft_c2c_2d_inverse_pass1(const fbfft_tensor* src, const fbfft_t
                        stream);
 }
 
-extern "C" size_t fbfft_make_tiles(const fbfft_tensor* input, const fbfft_tensor* output, int kH,
-                                   int kW, int fftSize, fbfft_tile* ins, fbfft_tile* outs,
-                                   size_t capacity) {
+extern "C" size_t fbfft_make_tiles_for_pass(int pass, const fbfft_tensor* input,
+                                            const fbfft_tensor* output, int kH, int kW,
+                                            int fftSize, fbfft_tile* ins, fbfft_tile* outs,
+                                            size_t capacity) {
   if (!okTensor(input, 4) || !okTensor(output, 4)) return 0;
+  if (pass < 0 || pass > 2) return 0;
   const int N = fftSize;
   if (!(N == 8 || N == 16 || N == 32) || kH < 1 || kW < 1 || kH > N || kW > N) return 0;
   const int H = input->size[2], W = input->size[3];
@@ -296,38 +318,71 @@ extern "C" size_t fbfft_make_tiles(const fbfft_tensor* input, const fbfft_tensor
   if (oH < 1 || oW < 1 || output->size[2] != oH || output->size[3] != oW) return 0;
   if (output->size[0] != input->size[0]) return 0;
   const int stepY = N - kH + 1, stepX = N - kW + 1;
-  const size_t ny = (size_t)ceilDiv(oH, stepY), nx = (size_t)ceilDiv(oW, stepX);
+  // updateOutput / accGradParameters walk the output in disjoint step x step windows;
+  // updateGradInput walks the input (the tensor it writes) in such windows
+  const bool byInput = pass == FBFFT_UPDATE_GRAD_INPUT;
+  const int spanY = byInput ? H : oH, spanX = byInput ? W : oW;
+  const size_t ny = (size_t)ceilDiv(spanY, stepY), nx = (size_t)ceilDiv(spanX, stepX);
   if (!ins || !outs) return ny * nx;
   size_t n = 0;
-  for (int y0 = 0; y0 < oH; y0 += stepY) {
-    for (int x0 = 0; x0 < oW; x0 += stepX, ++n) {
+  for (int y0 = 0; y0 < spanY; y0 += stepY) {
+    for (int x0 = 0; x0 < spanX; x0 += stepX, ++n) {
       if (n >= capacity) continue;
       fbfft_tile& ti = ins[n];
       fbfft_tile& to = outs[n];
-      ti.padL = ti.padU = to.padL = to.padU = 0;
-      ti.data = input->data + (size_t)y0 * input->stride[2] + (size_t)x0 * input->stride[3];
-      to.data = output->data + (size_t)y0 * output->stride[2] + (size_t)x0 * output->stride[3];
       for (int d = 0; d < 4; ++d) {
         ti.stride[d] = input->stride[d];
         to.stride[d] = output->stride[d];
       }
       ti.size[0] = input->size[0];
       ti.size[1] = input->size[1];
-      ti.size[2] = std::min(N, H - y0);
-      ti.size[3] = std::min(N, W - x0);
       to.size[0] = output->size[0];
       to.size[1] = output->size[1];
-      to.size[2] = std::min(stepY, oH - y0);
-      to.size[3] = std::min(stepX, oW - x0);
+      int iy = y0, ix = x0, oy = y0, ox = x0;  // window origins in input / output
+      if (!byInput) {
+        ti.padL = ti.padU = to.padL = to.padU = 0;
+        ti.size[2] = std::min(N, H - y0);
+        ti.size[3] = std::min(N, W - x0);
+        to.size[2] = std::min(stepY, oH - y0);
+        to.size[3] = std::min(stepX, oW - x0);
+      } else {
+        // gradInput rows y0 .. y0+step-1 are a full convolution over gradOutput rows
+        // y0-(kH-1) .. y0+step-1: N rows, placed from row 0 of the FFT plane (rows
+        // above the tensor's first stay zero through padU, rows below its last through
+        // the clipped size); the result for gradInput row y0 then sits in plane row
+        // kH-1, clear of the circular wrap-around, which the destination's pads skip.
+        oy = std::max(0, y0 - (kH - 1));
+        ox = std::max(0, x0 - (kW - 1));
+        to.padU = oy - (y0 - (kH - 1));
+        to.padL = ox - (x0 - (kW - 1));
+        to.size[2] = std::min(oH, y0 + stepY) - oy;
+        to.size[3] = std::min(oW, x0 + stepX) - ox;
+        ti.padU = kH - 1;
+        ti.padL = kW - 1;
+        ti.size[2] = std::min(stepY, H - y0);
+        ti.size[3] = std::min(stepX, W - x0);
+      }
+      ti.data = input->data + (size_t)iy * input->stride[2] + (size_t)ix * input->stride[3];
+      to.data = output->data + (size_t)oy * output->stride[2] + (size_t)ox * output->stride[3];
     }
   }
   return n;
+}
+
+extern "C" size_t fbfft_make_tiles(const fbfft_tensor* input, const fbfft_tensor* output, int kH,
+                                   int kW, int fftSize, fbfft_tile* ins, fbfft_tile* outs,
+                                   size_t capacity) {
+  return fbfft_make_tiles_for_pass(FBFFT_UPDATE_OUTPUT, input, output, kH, kW, fftSize, ins, outs,
+                                   capacity);
 }
 
 extern "C" int fbfft_iterated_conv(int fftSize, const fbfft_tile* ins, const fbfft_tile* outs,
                                    const fbfft_tensor* weight, int pass, float scale,
                                    int batchSize, size_t numTiles, fbfft_stream_t stream) {
   if (!okTensor(weight, 4) || !ins || !outs) return 0;
+  // a filter larger than the transform has no circular-convolution meaning; the
+  // windowed loader would silently drop its rows / columns beyond fftSize
+  if (weight->size[2] > fftSize || weight->size[3] > fftSize) return 0;
   return launchIteratedConv(fftSize, ins, outs, weight->data, weight->stride, weight->size, pass,
                             scale, batchSize, numTiles, stream);
 }

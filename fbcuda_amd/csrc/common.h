@@ -31,8 +31,10 @@ inline int ceilDiv(int a, int b) { return (a + b - 1) / b; }
 
 inline bool aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
 
+// status of the launches just made; the error is consumed, so that one failed
+// launch does not make every later call of the process report failure
 inline int launchStatus() {
-  return hipPeekAtLastError() == hipSuccess ? FBFFT_SUCCESS : FBFFT_HIP_ERROR;
+  return hipGetLastError() == hipSuccess ? FBFFT_SUCCESS : FBFFT_HIP_ERROR;
 }
 
 // kernel launchers implemented in the .hip files (return an fbfft_error)

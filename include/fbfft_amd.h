@@ -77,7 +77,8 @@ int fbfft_c2r_1d(const fbfft_tensor* real, const fbfft_tensor* cplx, int padL,
 
 /* fbfft2D<1>(real, complexAsFloat, padL, padU) (fbfft/FBFFT.cuh:30-36,
  * fbfft/FBFFT2D-inl.cuh:450-623).
- * real [B][h][w] is placed at (padU, padL) of a zero N x N plane.
+ * real [B][h][w] is placed at (padU, padL) of a zero N x N plane (h = 0 or w = 0
+ * with B > 0: the spectra are written as zeros).
  *   cplx [B][N/2+1][N][2], N in {8,16,32}:  cplx[b][ky][kx]  (one kernel)
  *   cplx [B][N/2+1][N][2], N in {64,128}:   cplx[b][kx][ky]  (one kernel; an
  *       extension: the reference needs two calls and a scratch buffer)
@@ -124,7 +125,8 @@ int fbfft_transpose_mm(const fbfft_tensor* A, const fbfft_tensor* B, const fbfft
 /* detail::FFTIteratedConvolution<FFTSize> (fbfft/FFTIteratedConvolution.cuh:624-755).
  * ins / outs are DEVICE pointers to numTiles descriptors each.  weight is
  * [Cout][Cin][kH][kW].  Returns 1 if a kernel was launched, 0 if the pass code or
- * FFT size matched nothing (the reference's bool), and a negative fbfft_error
+ * FFT size matched nothing (the reference's bool) or the filter is larger than
+ * the transform (kH or kW > fftSize), and a negative fbfft_error
  * (-FBFFT_HIP_ERROR ...) on launch failure.  FBFFT_ACC_GRAD_PARAMETERS overwrites
  * weight with scale * gradient; partial sums of several workgroups meet in atomic
  * adds, so its last bits can differ from run to run. */
@@ -143,9 +145,25 @@ int fbfft_iterated_conv(int fftSize, const fbfft_tile* ins, const fbfft_tile* ou
  * capacity descriptors into the HOST arrays ins / outs, which the caller then
  * copies to the device, and returns the number of tiles of the grid; with
  * ins == NULL or outs == NULL it only returns that number.  0 = unsupported
- * arguments.  The same descriptor arrays serve all three passes. */
+ * arguments.  This grid serves FBFFT_UPDATE_OUTPUT and FBFFT_ACC_GRAD_PARAMETERS.
+ * It does NOT serve FBFFT_UPDATE_GRAD_INPUT: that pass stores (does not add)
+ * each tile's result into ins[tile], and these input windows overlap by kH-1
+ * rows and kW-1 columns. */
 size_t fbfft_make_tiles(const fbfft_tensor* input, const fbfft_tensor* output, int kH, int kW,
                         int fftSize, fbfft_tile* ins, fbfft_tile* outs, size_t capacity);
+
+/* The same builder for a named pass.  pass = FBFFT_UPDATE_OUTPUT or
+ * FBFFT_ACC_GRAD_PARAMETERS gives the grid of fbfft_make_tiles.
+ * pass = FBFFT_UPDATE_GRAD_INPUT (input = gradInput, output = gradOutput) cuts
+ * gradInput into DISJOINT windows of (fftSize-kH+1) x (fftSize-kW+1), clipped at
+ * the edges, with padU = kH-1 and padL = kW-1, each paired with the gradOutput
+ * window of up to fftSize x fftSize that starts kH-1 rows above and kW-1 columns
+ * left of it (clipped at the tensor's edges; the clipped-off rows and columns
+ * become its padU / padL), so that every gradInput element is written by exactly
+ * one tile.  The tile count can differ from the other passes' count. */
+size_t fbfft_make_tiles_for_pass(int pass, const fbfft_tensor* input, const fbfft_tensor* output,
+                                 int kH, int kW, int fftSize, fbfft_tile* ins, fbfft_tile* outs,
+                                 size_t capacity);
 
 /* FFT convolution layer on the split path: the FFT -> transposeMM -> IFFT
  * sequences that the reference's external callers compose from the primitives

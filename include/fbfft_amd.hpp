@@ -255,14 +255,18 @@ bool FFTIteratedConvolution(TiledDeviceTensor<float, 4>* ins, TiledDeviceTensor<
 }
 
 // Host-side tile grid for FFTIteratedConvolution<FFTSize>: fills ins / outs (host
-// arrays of capacity descriptors) and returns the tile count; see fbfft_make_tiles.
+// arrays of capacity descriptors) and returns the tile count; see
+// fbfft_make_tiles_for_pass.  FFT_UpdateGradInput needs its own grid (disjoint
+// gradInput windows); the other two passes share one.
 template <int FFTSize>
 size_t makeTiles(const DeviceTensor<float, 4>& input, const DeviceTensor<float, 4>& output, int kH,
                  int kW, TiledDeviceTensor<float, 4>* ins, TiledDeviceTensor<float, 4>* outs,
-                 size_t capacity) {
+                 size_t capacity,
+                 FFTConvolutionPassFFI pass = FFTConvolutionPassFFI{FBFFT_UPDATE_OUTPUT}) {
   fbfft_tensor i = fbfft_amd_detail::describe(input), o = fbfft_amd_detail::describe(output);
-  return fbfft_make_tiles(&i, &o, kH, kW, FFTSize, reinterpret_cast<fbfft_tile*>(ins),
-                          reinterpret_cast<fbfft_tile*>(outs), capacity);
+  return fbfft_make_tiles_for_pass(pass.pass, &i, &o, kH, kW, FFTSize,
+                                   reinterpret_cast<fbfft_tile*>(ins),
+                                   reinterpret_cast<fbfft_tile*>(outs), capacity);
 }
 
 }  // namespace detail

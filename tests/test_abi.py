@@ -158,3 +158,51 @@ def test_make_tiles_capacity_and_rejects():
     assert F.lib().fbfft_conv_workspace(0, 4, 5, 6, 64) == (20 + 30 + 24) * 33 * 64 * 8
     assert F.lib().fbfft_conv_workspace(2, 4, 5, 6, 128) == (20 + 30 + 24) * 65 * 128 * 8 + 30 * 128 * 128 * 4
     assert F.lib().fbfft_conv_workspace(0, 4, 5, 6, 256) == 0
+
+
+def _descriptor_views(tiles, base_ptr, strides):
+    """(y0, x0, h, w, padL, padU) of each descriptor, recovered from its address."""
+    out = []
+    for t in tiles:
+        off = (t.data - base_ptr) // 4
+        assert (t.data - base_ptr) % 4 == 0 and off >= 0
+        y0, x0 = off // strides[2], off % strides[2]
+        out.append((y0, x0, t.size[2], t.size[3], t.padL, t.padU))
+    return out
+
+
+@pytest.mark.parametrize("N,kH,kW,H,W", [(8, 3, 3, 14, 17), (16, 5, 3, 30, 41), (32, 9, 9, 70, 56),
+                                         (8, 1, 1, 9, 9), (16, 16, 16, 16, 16), (8, 3, 2, 8, 6)])
+def test_grad_input_tile_grid_partitions_and_reproduces_gradient(oracle, N, kH, kW, H, W):
+    """fbfft_make_tiles_for_pass(FFT_UpdateGradInput) is host code: its gradInput windows
+    tile the tensor exactly once, and the CPU transcription of the tiled pass run over its
+    descriptors gives the fp64 input gradient (multi-tile, seams included)."""
+    import torch
+    from fbcuda_amd import synth
+    Nb, Cin, Cout = 2, 3, 2
+    gin = np.full((Nb, Cin, H, W), 7.0, np.float32)
+    g = synth.normal((Nb, Cout, H - kH + 1, W - kW + 1), seed=60).numpy()
+    w = synth.normal((Cout, Cin, kH, kW), seed=61, std=0.05).numpy()
+    vi, vo = F.view(torch.from_numpy(gin)), F.view(torch.from_numpy(g))
+    n = F.lib().fbfft_make_tiles_for_pass(1, vi, vo, kH, kW, N, None, None, 0)
+    stepY, stepX = N - kH + 1, N - kW + 1
+    assert n == -(-H // stepY) * -(-W // stepX)
+    a, b = (F.Tile * n)(), (F.Tile * n)()
+    assert F.lib().fbfft_make_tiles_for_pass(1, vi, vo, kH, kW, N, ctypes.cast(a, ctypes.c_void_p),
+                                             ctypes.cast(b, ctypes.c_void_p), n) == n
+    iv = _descriptor_views(a, gin.ctypes.data, [s // 4 for s in gin.strides])
+    ov = _descriptor_views(b, g.ctypes.data, [s // 4 for s in g.strides])
+    cover = np.zeros((H, W), np.int32)
+    for (y0, x0, h, wd, padL, padU), (gy, gx, gh, gw, gpl, gpu) in zip(iv, ov):
+        cover[y0:y0 + h, x0:x0 + wd] += 1
+        assert (padU, padL) == (kH - 1, kW - 1) and h >= 1 and wd >= 1
+        assert gh >= 1 and gw >= 1 and gpu + gh <= N and gpl + gw <= N
+        assert gy - gpu == y0 - (kH - 1) and gx - gpl == x0 - (kW - 1)
+    assert (cover == 1).all()
+    assert oracle.iterated_conv(N, gin, iv, g.copy(), ov, w, 1) == 1
+    from oracle import rel_l2
+    assert rel_l2(gin, oracle.corr2d_grad_input(g, w, H, W)) < 1e-4
+    # passes 0 and 2 share the grid of fbfft_make_tiles
+    assert F.lib().fbfft_make_tiles_for_pass(2, vi, vo, kH, kW, N, None, None, 0) == \
+        F.lib().fbfft_make_tiles(vi, vo, kH, kW, N, None, None, 0)
+    assert F.lib().fbfft_make_tiles_for_pass(3, vi, vo, kH, kW, N, None, None, 0) == 0

@@ -65,12 +65,22 @@ def test_three_passes_vs_oracle(oracle, N, k, H, W, Nb, Cin, Cout):
     assert rel(gw, gw_want) < TOL_CONV
     assert rel(gw, 0.5 * oracle.corr2d_grad_weight(x, g, k, k)) < TOL_CONV
 
-    # updateGradInput: every tile writes (not accumulates) its N x N input window,
-    # exactly as the reference does; compare with the transcription tile for tile
-    gin0 = np.full_like(x, 7.0)
-    launched, gin, _, _ = run_pass(N, gin0, iv, g, ov, w, F.FFT_UpdateGradInput)
-    assert launched
+    # updateGradInput stores (does not accumulate) each tile's result, as the reference
+    # does, so it runs on its own grid: disjoint gradInput windows with pads kH-1 / kW-1,
+    # each fed by the N x N gradOutput window around it (fbfft_make_tiles_for_pass)
+    d = dev()
+    gin_d = torch.full(x.shape, 7.0, device=d)
+    g_d, w_d = torch.from_numpy(g).to(d), torch.from_numpy(w).to(d)
+    bins, bouts, nb = F.make_tile_grid(gin_d, g_d, k, k, N, F.FFT_UpdateGradInput)
+    assert nb == -(-H // (N - k + 1)) * -(-W // (N - k + 1))
+    assert F.FFTIteratedConvolution(N, bins, bouts, w_d, F.FFT_UpdateGradInput, 1.0, Nb, nb)
+    torch.cuda.synchronize()
+    assert rel(gin_d.cpu().numpy(), oracle.corr2d_grad_input(g, w, H, W)) < TOL_CONV
+    # the overlapping grid of the other passes is only defined for a single tile
     if len(iv) == 1:
+        gin0 = np.full_like(x, 7.0)
+        launched, gin, _, _ = run_pass(N, gin0, iv, g, ov, w, F.FFT_UpdateGradInput)
+        assert launched
         gin_want = gin0.copy()
         assert oracle.iterated_conv(N, gin_want, iv, g.copy(), ov, w, 1) == 1
         assert rel(gin, gin_want) < TOL_CONV
@@ -168,8 +178,8 @@ def test_library_tile_grid_matches_reference_tiling(oracle):
 
 @pytest.mark.parametrize("seed", range(16))
 def test_random_tilings(oracle, seed):
-    """updateOutput and accGradParameters on a seeded random image / filter / plane
-    count with the library's own tile grid, against fp64 direct correlation."""
+    """All three passes on a seeded random image / filter / plane count with the
+    library's own tile grids, against fp64 direct correlation and its gradients."""
     rng = np.random.default_rng(5000 + seed)
     N = int(rng.choice([8, 16, 32]))
     k = int(rng.integers(1, min(N - 1, 9) + 1))
@@ -191,3 +201,8 @@ def test_random_tilings(oracle, seed):
     assert F.FFTIteratedConvolution(N, gins, gouts, gw, F.FFT_AccGradParameters, 0.25, Nb, n2), tag
     torch.cuda.synchronize()
     assert rel(gw.cpu().numpy(), 0.25 * oracle.corr2d_grad_weight(xh, g.cpu().numpy(), k, k)) < TOL_CONV, tag
+    gin = torch.full_like(x, float("nan"))
+    bins, bouts, n3 = F.make_tile_grid(gin, g, k, k, N, F.FFT_UpdateGradInput)
+    assert F.FFTIteratedConvolution(N, bins, bouts, w, F.FFT_UpdateGradInput, 1.0, Nb, n3), tag
+    torch.cuda.synchronize()
+    assert rel(gin.cpu().numpy(), oracle.corr2d_grad_input(g.cpu().numpy(), wh, H, W)) < TOL_CONV, tag
