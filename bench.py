@@ -50,6 +50,25 @@ def timed(fn, steps, warmup, torch):
     return (t1 - t0) / steps, e0.elapsed_time(e1) * 1e-3 / steps
 
 
+def spread(fn, steps, torch, chunks=20):
+    """Median and minimum seconds per launch over `chunks` consecutive groups of at least
+    five launches, each group bracketed by its own pair of HIP events (a separate pass
+    after the timed region, so that the extra events do not sit inside it; an event
+    around every single launch would add 2-3 us to a 22 us kernel)."""
+    n = chunks
+    per = max(5, steps // n)
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(n + 1)]
+    ev[0].record()
+    for c in range(n):
+        for _ in range(per):
+            fn()
+        ev[c + 1].record()
+    torch.cuda.synchronize()
+    ts = sorted(ev[c].elapsed_time(ev[c + 1]) * 1e-3 / per for c in range(n))
+    mid = ts[n // 2] if n % 2 else 0.5 * (ts[n // 2 - 1] + ts[n // 2])
+    return mid, ts[0]
+
+
 def prepared(fn_name, F, *tensors_then_ints):
     """Bind a C-ABI call once: descriptors are built outside the timed region."""
     import torch
@@ -75,9 +94,38 @@ def prepared(fn_name, F, *tensors_then_ints):
     return call
 
 
+NATIVE_FLAGS = ["-O3", "-march=native", "-std=c++17", "-fPIC", "-fopenmp", "-ffp-contract=off",
+                "-fno-fast-math"]
+
+
+def native_oracle():
+    """The CPU oracle compiled for THIS machine's cores (-O3 -march=native, contraction
+    off) into a temporary directory; the in-tree library is built on another machine with
+    a portable -march and is what is used when no compiler is at hand.  Returns
+    (module, flags string)."""
+    import shutil
+    import subprocess
+    import tempfile
+
+    import oracle as O
+    cxx = shutil.which("g++")
+    src = os.path.join(ROOT, "oracle", "fbfft_oracle.cpp")
+    if cxx and os.path.exists(src):
+        out = os.path.join(tempfile.mkdtemp(prefix="fbfft_oracle_"), "liboracle_native.so")
+        try:
+            subprocess.check_call([cxx] + NATIVE_FLAGS + ["-shared", "-o", out, src],
+                                  stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL, timeout=120)
+            O.use_library(out)
+            return O, " ".join(NATIVE_FLAGS[:2]) + " -ffp-contract=off, built on this machine"
+        except (subprocess.SubprocessError, OSError):
+            pass
+    O.lib()
+    return O, "in-tree build (oracle/Makefile flags)"
+
+
 def cpu_baseline(x_host, N, budget_s=12.0):
     """Times the CPU oracle (kind "port") on the same planes; bounded to ~budget_s."""
-    import oracle as O
+    O, flags = native_oracle()
     threads = O.num_threads()
     O.fbfft2d(x_host[:64], N)  # warm
     t0 = time.perf_counter()
@@ -99,19 +147,29 @@ def cpu_baseline(x_host, N, budget_s=12.0):
     return {"value": round(gbs, 3), "unit": "GB/s", "cores": threads, "kind": "port",
             "sample": "%d passes of the full %d-plane %dx%d R2C batch, OpenMP over planes, "
                       "%.3f s per pass" % (reps, x_host.shape[0], N, N, dt),
+            "flags": flags,
             "single_thread_GBps": round(x_host.shape[0] * plane_bytes(N) / dt1 / 1e9, 3)}
+
+
+def profile_figure(name, key):
+    """An integer `key: value` line of a committed rocprofv3 summary under profiles/, or None."""
+    try:
+        for line in open(os.path.join(ROOT, "profiles", name)):
+            if line.startswith(key + ":"):
+                return int(line.split(":")[1])
+    except (OSError, ValueError):
+        pass
+    return None
 
 
 def measured_traffic():
     """HBM bytes per R2C launch from the committed rocprofv3 counter summary, or None."""
-    path = os.path.join(ROOT, "profiles", "fft2dSmallForward32_configs1.md")
-    try:
-        for line in open(path):
-            if line.startswith("traffic_bytes_per_launch:"):
-                return int(line.split(":")[1])
-    except OSError:
-        pass
-    return None
+    return profile_figure("fft2dSmallForward32_configs1.md", "traffic_bytes_per_launch")
+
+
+MFMA_FP32_PEAK = 157.3e12
+CONV3_FLOP = 544 * 128 * 192 * 64 * 8.0          # 8 flop per complex multiply-add
+CONV3_FLOP_ISSUED = 544 * 128 * 192 * 64 * 6.0   # three real products per complex product
 
 
 def conv_extras(F, synth, torch, dev, extra):
@@ -131,9 +189,23 @@ def conv_extras(F, synth, torch, dev, extra):
         if rc != 0:
             raise RuntimeError(F.error_string(rc))
     _, t = timed(conv, 200, 200, torch)
+    mid, low = spread(conv, 200, torch)
     extra["fft_conv_configs3_ms_per_iter"] = round(t * 1e3, 4)
+    extra["fft_conv_configs3_ms_per_iter_median"] = round(mid * 1e3, 4)
+    extra["fft_conv_configs3_ms_per_iter_min"] = round(low * 1e3, 4)
     extra["fft_conv_configs3_direct_equiv_TFLOPs"] = round(41.6e9 / t / 1e12, 1)
     extra["fft_conv_configs3_fp32_peak_direct_ms"] = round(41.6e9 / 157.3e12 * 1e3, 4)
+    # the second half of the metric against its roofline: the whole iteration (forward
+    # transforms, contraction, inverse transform) is charged to the contraction's matrix
+    # work, 8 flop per complex multiply-add; frac_issued counts the 6 flop the kernels issue
+    extra["fft_conv_roofline"] = {
+        "bound": "mfma", "achieved": round(CONV3_FLOP / t / 1e12, 2), "peak": MFMA_FP32_PEAK / 1e12,
+        "unit": "TFLOP/s", "frac": round(CONV3_FLOP / t / MFMA_FP32_PEAK, 4),
+        "frac_issued": round(CONV3_FLOP_ISSUED / t / MFMA_FP32_PEAK, 4),
+        "floor_us": round(CONV3_FLOP / MFMA_FP32_PEAK * 1e6, 1), "iter_us": round(t * 1e6, 1),
+        "traffic": profile_figure("conv_pipeline_configs3.md", "traffic_bytes_per_iteration"),
+        "algorithmic_bytes": 77119488,
+        "workload": "configs[3]: 128x64x27x27 * 192x64x5x5 -> 128x192x23x23, 32-point FFTs"}
     # the other two passes of the same layer
     g = synth.normal((128, 192, 23, 23), seed=32, device=dev)
     gi, gw = torch.empty_like(x), torch.empty_like(w)
@@ -314,9 +386,44 @@ def main():
     inv = prepared("fbfft_c2r_2d", F, spec, back, 0, 0)
 
     step_s, launch_s = timed(fwd, args.steps, args.warmup, torch)
+    launch_mid, launch_min = spread(fwd, args.steps, torch)
     nbytes = B * plane_bytes(N)
     value = nbytes / step_s / 1e9
-    achieved = nbytes / launch_s / 1e9
+
+    def hbm_roofline(nb, t, mid, low, note):
+        return {"bound": "hbm", "achieved": round(nb / t / 1e9, 1), "peak": HBM_PEAK_GBS,
+                "unit": "GB/s", "frac": round(nb / t / 1e9 / HBM_PEAK_GBS, 4),
+                "frac_median": round(nb / mid / 1e9 / HBM_PEAK_GBS, 4),
+                "frac_best": round(nb / low / 1e9 / HBM_PEAK_GBS, 4),
+                "kernel": "fft2dSmallForward<32>", "bytes_per_launch": nb,
+                "launch_us": round(t * 1e6, 2), "launch_us_median": round(mid * 1e6, 2),
+                "launch_us_min": round(low * 1e6, 2), "residency": note}
+
+    # configs[1]'s 132 MB of operands fit the 256 MiB last-level cache when the same
+    # buffers are used launch after launch.  Two measurements whose operands come from
+    # HBM: the same 16384-plane launch rotating over four distinct buffer sets (528 MB),
+    # and one launch over a 4x batch.
+    sets = [(x, spec)]
+    for i in range(3):
+        sets.append((synth.normal((B, N, N), seed=100 + i, device=dev), torch.empty_like(spec)))
+    calls = [prepared("fbfft_r2c_2d", F, a, b, 0, 0) for a, b in sets]
+    turn = [0]
+
+    def rotating():
+        calls[turn[0] & 3]()
+        turn[0] += 1
+    _, rot_s = timed(rotating, max(args.steps, 40), max(args.warmup, 8), torch)
+    rot_mid, rot_min = spread(rotating, max(args.steps, 40), torch)
+    roofline_rotating = hbm_roofline(nbytes, rot_s, rot_mid, rot_min,
+                                     "hbm: configs[1] launches rotate over 4 buffer sets, 528 MB")
+    del sets, calls
+    x4 = synth.normal((4 * B, N, N), seed=6, device=dev)
+    s4 = torch.empty((4 * B, N // 2 + 1, N, 2), device=dev)
+    f4 = prepared("fbfft_r2c_2d", F, x4, s4, 0, 0)
+    _, l4 = timed(f4, max(20, args.steps // 4), max(args.warmup // 4, 5), torch)
+    m4, b4 = spread(f4, max(20, args.steps // 4), torch)
+    roofline_4x = hbm_roofline(4 * nbytes, l4, m4, b4, "hbm: one launch over 65536 planes, 554 MB")
+    del x4, s4, f4
 
     extra = {}
     if not args.no_extra:
@@ -325,7 +432,7 @@ def main():
         # round-trip sanity on the benchmark tensors themselves
         err = float((back / (N * N) - x).double().norm() / x.double().norm())
         extra["roundtrip_rel_l2"] = err
-        for n2, b2 in ((32, 65536), (16, 262144), (8, 1048576), (64, 16384), (128, 4096)):
+        for n2, b2 in ((16, 262144), (8, 1048576), (64, 16384), (128, 4096)):
             x2 = synth.normal((b2, n2, n2), seed=2 + n2.bit_length() - 1, device=dev)
             s2 = torch.empty((b2, n2 // 2 + 1, n2, 2), device=dev)
             f2 = prepared("fbfft_r2c_2d", F, x2, s2, 0, 0)
@@ -368,10 +475,11 @@ def main():
         "data": "synthetic",
         "config": {"workload": "configs[1]: fbfft2D R2C, 16384 planes of 32x32 fp32 N(0,1) seed 1, "
                                "output [16384][17][32][2]; 8448 algorithmic bytes per plane"},
-        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": measured_traffic(),
-                     "kernel": "fft2dSmallForward<32>", "bytes_per_launch": nbytes,
-                     "launch_us": round(launch_s * 1e6, 2)},
+        "roofline": dict(hbm_roofline(nbytes, launch_s, launch_mid, launch_min,
+                                      "last-level cache: the same 132 MB of operands every launch"),
+                         traffic=measured_traffic()),
+        "roofline_rotating": roofline_rotating,
+        "roofline_4x": roofline_4x,
         "extra": extra,
     }
     if not args.no_cpu:

@@ -33,6 +33,15 @@ def lib():
     return _lib
 
 
+def use_library(path):
+    """Load the oracle from another build of fbfft_oracle.cpp (bench.py's cpu_baseline
+    compiles one for the machine it runs on)."""
+    global _lib
+    _lib = ctypes.CDLL(path)
+    _lib.orc_num_threads.restype = ctypes.c_int
+    return _lib
+
+
 def _f32(a):
     return np.ascontiguousarray(a, dtype=np.float32)
 

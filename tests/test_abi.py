@@ -206,3 +206,22 @@ def test_grad_input_tile_grid_partitions_and_reproduces_gradient(oracle, N, kH, 
     assert F.lib().fbfft_make_tiles_for_pass(2, vi, vo, kH, kW, N, None, None, 0) == \
         F.lib().fbfft_make_tiles(vi, vo, kH, kW, N, None, None, 0)
     assert F.lib().fbfft_make_tiles_for_pass(3, vi, vo, kH, kW, N, None, None, 0) == 0
+
+
+def test_view_rejects_strides_beyond_32_bits():
+    import torch
+    t = torch.empty(4).as_strided((1, 2), (2 ** 31, 1))
+    with pytest.raises(ValueError):
+        F.view(t)
+    assert F.view(torch.empty(4).as_strided((1, 2), (2 ** 31 - 1, 1))).stride[0] == 2 ** 31 - 1
+
+
+def test_iterated_conv_refuses_filters_larger_than_the_transform():
+    """Validated on the host before anything is launched: returns 0 (not launched)."""
+    import torch
+    w = torch.zeros((1, 1, 9, 3))
+    ins, outs = (F.Tile * 1)(), (F.Tile * 1)()
+    rc = F.lib().fbfft_iterated_conv(8, ctypes.cast(ins, ctypes.c_void_p),
+                                     ctypes.cast(outs, ctypes.c_void_p), F.view(w), 0,
+                                     ctypes.c_float(1.0), 1, 1, None)
+    assert rc == 0

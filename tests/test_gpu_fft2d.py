@@ -260,3 +260,14 @@ def test_odd_plane_stride_mixes_the_window_load_paths(oracle, N):
     assert F.fbifft2D(spec, back, 2, 1) == F.Success
     torch.cuda.synchronize()
     assert rel(back.cpu().numpy(), N * N * x.astype(np.float64)) < TOL_FFT
+
+
+@pytest.mark.parametrize("N", [4, 8, 32, 64])
+@pytest.mark.parametrize("h,w", [(0, 3), (3, 0)])
+def test_empty_window_gives_zero_spectra(N, h, w):
+    """B > 0 planes whose real window is empty are all padding: zeros, not stale data."""
+    x = torch.zeros((3, h, w), device=dev())
+    out = torch.full((3, N // 2 + 1, N, 2), float("nan"), device=dev())
+    assert F.fbfft2D(x, out) == F.Success
+    torch.cuda.synchronize()
+    assert float(out.abs().max()) == 0.0

@@ -62,6 +62,36 @@ def test_mm_vs_oracle(oracle, conjA, conjB, I, J, K, shape):
     assert rel(acc.reshape(I, J, xy, 2), want_acc) < TOL_FFT
 
 
+@pytest.mark.parametrize("conjA,conjB", ROLES)
+def test_mm_cancellation_per_element(oracle, conjA, conjB):
+    """The contraction forms a complex product from three real products; its imaginary
+    and real parts are differences of larger terms.  Operands with |re| close to |im| and
+    a long reduction make those differences cancel: every element must stay within a
+    bound relative to sum_k (|a_re|+|a_im|)(|b_re|+|b_im|), not just in the norm."""
+    I, J, K, xy = 40, 24, 512, 12
+    rng = np.random.default_rng(77)
+
+    def near_diagonal(shape):
+        mag = rng.uniform(0.5, 2.0, shape) * rng.choice([-1.0, 1.0], shape)
+        eps = rng.uniform(-1e-3, 1e-3, shape)
+        return np.stack([mag, mag * (1.0 + eps)], axis=-1).astype(np.float32)
+
+    A = near_diagonal(((K, I) if conjA else (I, K)) + (xy,))
+    B = near_diagonal(((J, K) if conjB else (K, J)) + (xy,))
+    rc, got = mm(A, B, conjA, conjB, 1.0)
+    assert rc == F.Success
+    want = oracle.transpose_mm64(A, B, conjA, conjB, 1.0)
+    absA = np.abs(A).sum(-1).astype(np.float64)
+    absB = np.abs(B).sum(-1).astype(np.float64)
+    a_ik = absA.transpose(1, 0, 2) if conjA else absA            # [I][K][xy]
+    b_kj = absB.transpose(1, 0, 2) if conjB else absB            # [K][J][xy]
+    scale = np.einsum("ikx,kjx->ijx", a_ik, b_kj)
+    eps32 = float(np.finfo(np.float32).eps)
+    bound = (K ** 0.5 + 8) * eps32 * scale
+    err = np.abs(got.astype(np.float64) - want).max(-1)
+    assert (err <= bound).all(), float((err / bound).max())
+
+
 def test_mm_empty_reduction():
     """K = 0: C = invNorm * (accumulate ? C : 0); the operands have no elements."""
     d = dev()
