@@ -46,7 +46,7 @@ _lib = None
 # every symbol include/fbfft_amd.h declares
 EXPORTS = (
     "fbfft_r2c_1d", "fbfft_c2r_1d", "fbfft_r2c_2d", "fbfft_c2c_2d_pass2", "fbfft_c2r_2d",
-    "fbfft_c2c_2d_inverse_pass1", "fbfft_transpose_mm", "fbfft_iterated_conv", "fbfft_make_tiles",
+    "fbfft_c2c_2d_inverse_pass1", "fbfft_transpose_mm", "fbfft_transpose_mm_packed", "fbfft_iterated_conv", "fbfft_make_tiles",
     "fbfft_make_tiles_for_pass",
     "fbfft_conv_workspace", "fbfft_conv_fprop_workspace", "fbfft_conv_fprop", "fbfft_conv_bprop",
     "fbfft_conv_accgrad", "fbfft_conv_fprop_static", "fbfft_error_string",
@@ -73,6 +73,7 @@ def lib():
         L.fbfft_c2c_2d_inverse_pass1.argtypes = [tp, tp, vp]
         L.fbfft_transpose_mm.argtypes = [tp, tp, tp, ctypes.c_int, ctypes.c_int, ctypes.c_int,
                                          ctypes.c_float, vp]
+        L.fbfft_transpose_mm_packed.argtypes = L.fbfft_transpose_mm.argtypes
         L.fbfft_iterated_conv.argtypes = [ctypes.c_int, vp, vp, tp, ctypes.c_int, ctypes.c_float,
                                           ctypes.c_int, ctypes.c_size_t, vp]
         L.fbfft_make_tiles.argtypes = [tp, tp, ctypes.c_int, ctypes.c_int, ctypes.c_int, vp, vp,
@@ -173,12 +174,16 @@ def fbifft2D_pass1(src, dst, stream=None):
 
 
 def transposeMM(A, B, C, invNorm, conjugateTransposeA=False, conjugateTransposeB=False,
-                accumulate=False, stream=None):
-    """transposeMM<Dim, ConjugateTransposeA, ConjugateTransposeB, Accumulate> (MM.cuh:11-17)."""
+                accumulate=False, stream=None, packed=False):
+    """transposeMM<Dim, ConjugateTransposeA, ConjugateTransposeB, Accumulate> (MM.cuh:11-17).
+
+    packed: operands are [d0][d1][N/2][N][2] spectra in the packed format of
+    fbfft2D (Unpack = false, fbfft/FFT2D32.cuh:421-427); row 0 is multiplied by the
+    unpack / multiply / re-pack rule of fbfft/FFTIteratedConvolution.cuh:161-186."""
     _on_gpu(A, B, C)
-    return lib().fbfft_transpose_mm(view(A), view(B), view(C), int(conjugateTransposeA),
-                                    int(conjugateTransposeB), int(accumulate), float(invNorm),
-                                    _stream(stream))
+    fn = lib().fbfft_transpose_mm_packed if packed else lib().fbfft_transpose_mm
+    return fn(view(A), view(B), view(C), int(conjugateTransposeA), int(conjugateTransposeB),
+              int(accumulate), float(invNorm), _stream(stream))
 
 
 def make_tiles(t, windows):

@@ -128,8 +128,11 @@ int fbfft_r2c_2d(const fbfft_tensor* real, const fbfft_tensor* cplx, int padL, i
   if (real->size[0] != cplx->size[0]) return FBFFT_UNSUPPORTED_DIMENSION;
   const int s1 = cplx->size[1], s2 = cplx->size[2];
   int N = 0;
-  bool scratchForm = false;
-  if ((s2 == 2 || s2 == 4 || s2 == 8 || s2 == 16 || s2 == 32 || s2 == 64 || s2 == 128) &&
+  bool scratchForm = false, packed = false;
+  if ((s2 == 8 || s2 == 16 || s2 == 32) && s1 == s2 / 2) {
+    N = s2;
+    packed = true;
+  } else if ((s2 == 2 || s2 == 4 || s2 == 8 || s2 == 16 || s2 == 32 || s2 == 64 || s2 == 128) &&
       s1 == s2 / 2 + 1) {
     N = s2;
   } else if ((s1 == 64 || s1 == 128) && s2 == s1 / 2 + 1) {
@@ -145,7 +148,8 @@ int fbfft_r2c_2d(const fbfft_tensor* real, const fbfft_tensor* cplx, int padL, i
   // B > 0 planes with an empty real window: every sample is padding
   if (empty(real)) return launchZeroSpectrum(cplxView4(cplx), stream);
   if (N < 8) return launchFft2dTinyForward(N, realView3(real), cplxView4(cplx), padL, padU, stream);
-  if (N <= 32) return launchFft2dSmallForward(N, realView3(real), cplxView4(cplx), padL, padU, stream);
+  if (N <= 32)
+    return launchFft2dSmallForward(N, realView3(real), cplxView4(cplx), padL, padU, stream, packed);
   if (!scratchForm)
     return launchFft2dLargeForward(N, realView3(real), cplxView4(cplx), padL, padU, stream);
   return launchTwoPass(N, 0, real->data, real->stride[0], real->stride[1], real->stride[2],
@@ -163,12 +167,14 @@ int fbfft_c2r_2d(const fbfft_tensor* cplx, const fbfft_tensor* real, int padL, i
     return FBFFT_UNSUPPORTED_SIZE;
   const bool half = (s1 == N / 2 + 1);
   const bool full = (N >= 64 && s1 == N);
-  if (!half && !full) return FBFFT_UNSUPPORTED_SIZE;
+  const bool packed = (N >= 8 && N <= 32 && s1 == N / 2);
+  if (!half && !full && !packed) return FBFFT_UNSUPPORTED_SIZE;
   if (padL < 0 || padU < 0) return FBFFT_UNSUPPORTED_SIZE;
   if (!okCplx(cplx)) return FBFFT_UNSUPPORTED_DIMENSION;
   if (empty(real) || empty(cplx)) return FBFFT_SUCCESS;
   if (N < 8) return launchFft2dTinyInverse(N, cplxView4(cplx), realView3(real), padL, padU, stream);
-  if (N <= 32) return launchFft2dSmallInverse(N, cplxView4(cplx), realView3(real), padL, padU, stream);
+  if (N <= 32)
+    return launchFft2dSmallInverse(N, cplxView4(cplx), realView3(real), padL, padU, stream, packed);
   if (half) return launchFft2dLargeInverse(N, cplxView4(cplx), realView3(real), padL, padU, stream);
   return launchTwoPass(N, 3, cplx->data, cplx->stride[0], cplx->stride[1], cplx->stride[2],
                        real->data, real->stride[0], real->stride[1], real->stride[2],
@@ -197,6 +203,31 @@ extern "C" int fbfft_transpose_mm(const fbfft_tensor* A, const fbfft_tensor* B,
   return launchTransposeMM(A->data, A->stride[0], A->stride[1], B->data, B->stride[0],
                            B->stride[1], C->data, C->stride[0], C->stride[1], I, J, K, xa,
                            conjA != 0, conjB != 0, accumulate != 0, invNorm, stream);
+}
+
+extern "C" int fbfft_transpose_mm_packed(const fbfft_tensor* A, const fbfft_tensor* B,
+                                         const fbfft_tensor* C, int conjA, int conjB,
+                                         int accumulate, float invNorm, fbfft_stream_t stream) {
+  if (!A || !B || !C) return FBFFT_UNSUPPORTED_DIMENSION;
+  if (conjA && conjB) return FBFFT_UNSUPPORTED_DIMENSION;
+  if (A->dim != 5 || B->dim != 5 || C->dim != 5) return FBFFT_UNSUPPORTED_DIMENSION;
+  const int N = A->size[3];
+  if (!(N == 8 || N == 16 || N == 32)) return FBFFT_UNSUPPORTED_SIZE;
+  const fbfft_tensor* ts[3] = {A, B, C};
+  for (const fbfft_tensor* t : ts) {
+    if (t->size[3] != N || t->size[2] != N / 2) return FBFFT_UNSUPPORTED_SIZE;
+    if (collapsedBins(t) != N / 2 * N) return FBFFT_UNSUPPORTED_DIMENSION;
+    if (t->stride[0] % 2 != 0 || t->stride[1] % 2 != 0 || !aligned(t->data, 8))
+      return FBFFT_UNSUPPORTED_DIMENSION;
+  }
+  const int I = conjA ? A->size[1] : A->size[0];
+  const int K = conjA ? A->size[0] : A->size[1];
+  const int Kb = conjB ? B->size[1] : B->size[0];
+  const int J = conjB ? B->size[0] : B->size[1];
+  if (K != Kb || C->size[0] != I || C->size[1] != J) return FBFFT_UNSUPPORTED_DIMENSION;
+  return launchTransposeMMPacked(A->data, A->stride[0], A->stride[1], B->data, B->stride[0],
+                                 B->stride[1], C->data, C->stride[0], C->stride[1], I, J, K, N,
+                                 conjA != 0, conjB != 0, accumulate != 0, invNorm, stream);
 }
 
 namespace {

@@ -39,9 +39,9 @@ inline int launchStatus() {
 
 // kernel launchers implemented in the .hip files (return an fbfft_error)
 int launchFft2dSmallForward(int N, const RealView& real, const CplxView& cplx, int padL, int padU,
-                            hipStream_t s);
+                            hipStream_t s, bool packed = false);
 int launchFft2dSmallInverse(int N, const CplxView& cplx, const RealView& real, int padL, int padU,
-                            hipStream_t s);
+                            hipStream_t s, bool packed = false);
 
 int launchFft2dTinyForward(int N, const RealView& real, const CplxView& cplx, int padL, int padU,
                            hipStream_t s);
@@ -59,6 +59,10 @@ int launchFft1d(bool forward, int N, float* real, int sb, int sx, float* cplx, i
 int launchTransposeMM(const float* A, long a0, long a1, const float* B, long b0, long b1, float* C,
                       long c0, long c1, int I, int J, int K, int XY, bool conjA, bool conjB,
                       bool accumulate, float invNorm, hipStream_t s);
+
+int launchTransposeMMPacked(const float* A, long a0, long a1, const float* B, long b0, long b1,
+                            float* C, long c0, long c1, int I, int J, int K, int N, bool conjA,
+                            bool conjB, bool accumulate, float invNorm, hipStream_t s);
 
 int launchIteratedConv(int N, const fbfft_tile* ins, const fbfft_tile* outs, float* weight,
                        const int* wStride, const int* wSize, int pass, float scale, int batch,

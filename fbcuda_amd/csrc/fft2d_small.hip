@@ -17,6 +17,11 @@
 //     16-byte stores per wave; rows 0 and N/2 are unpacked on the way out.
 // The inverse runs the same steps backwards.  Each plane crosses HBM exactly
 // once in each direction: 4N^2 + 8N(N/2+1) bytes.
+//
+// PACKED variants keep the reference's packed spectrum format (the Unpack = false
+// store of fbfft/FFT2D32.cuh:421-427 and the PackedInput = true core of :302-316):
+// cplx is [B][N/2][N][2] and its row 0 holds F[0][kx] + i F[N/2][kx], the form the
+// row travels in inside the kernel anyway, so the copy stages move N/2 plain rows.
 #include "common.h"
 #include "fft2d_core.h"
 #include "fft_regs.h"
@@ -24,14 +29,14 @@
 namespace fbfft_amd {
 namespace {
 
-template <int N>
+template <int N, bool PACKED = false>
 struct SmallCfg {
   static constexpr int H = N / 2;
   static constexpr int T = N / 2;          // lanes per plane
   static constexpr int P = 64 / T;         // planes per wave
-  static constexpr int ROWS = H + 1;       // spectral rows kept in LDS
+  static constexpr int ROWS = PACKED ? H : H + 1;  // spectral rows of a plane in memory
   static constexpr int RS = PlaneCfg<N>::RS;  // LDS row stride (complex)
-  static constexpr int PS = ROWS * RS + (N == 8 ? 2 : 0);  // LDS plane stride (complex)
+  static constexpr int PS = (H + 1) * RS + (N == 8 ? 2 : 0);  // LDS plane stride (complex)
   static constexpr int F4_PER_PLANE = ROWS * N / 2;        // float4 per spectrum plane
   static constexpr int ITERS = P * F4_PER_PLANE / 64;      // float4 per lane per wave
   static_assert(P * F4_PER_PLANE % 64 == 0, "copy loop must divide evenly");
@@ -45,10 +50,10 @@ struct SmallCfg {
 //            the second group are issued as soon as the first group's columns
 //            have left the registers, so they fly under the first group's row
 //            pass and stores: the wave pays the HBM latency once instead of twice.
-template <int N, bool FAST_REAL, bool FAST_CPLX, int GPW>
+template <int N, bool FAST_REAL, bool FAST_CPLX, int GPW, bool PACKED>
 __global__ __launch_bounds__(64) void fft2dSmallForward(RealView real, CplxView cplx, int padL,
                                                         int padU) {
-  using C = SmallCfg<N>;
+  using C = SmallCfg<N, PACKED>;
   constexpr int H = C::H, T = C::T, P = C::P, RS = C::RS, PS = C::PS;
   __shared__ __align__(16) c32 lds[P * PS];
 
@@ -86,8 +91,8 @@ __global__ __launch_bounds__(64) void fft2dSmallForward(RealView real, CplxView 
       // them is row 0 or N/2 of a plane (12 of the 17 iterations at N = 32) plane and
       // row are compile-time constants plus the lane's row within the iteration.
       constexpr int RPI = 64 / (N / 2);
-      constexpr int R0 = RPI * t, pp0 = R0 / (H + 1), r0 = R0 % (H + 1);
-      if constexpr (r0 >= 1 && r0 + RPI - 1 <= H - 1) {
+      constexpr int R0 = RPI * t, pp0 = R0 / C::ROWS, r0 = R0 % C::ROWS;
+      if constexpr ((PACKED || r0 >= 1) && r0 + RPI - 1 <= H - 1) {
         const int g = lane / (N / 2), xq = lane % (N / 2);
         const float4 v = ldsLoad4(lds + pp0 * PS + (r0 + g) * RS + 2 * xq);
         const int bo = b0 + pp0;
@@ -110,7 +115,7 @@ __global__ __launch_bounds__(64) void fft2dSmallForward(RealView real, CplxView 
       const int kx = 2 * (rem % (N / 2));
       const c32* base = lds + pp * PS;
       float4 v;
-      if (r == 0 || r == H) {
+      if (!PACKED && (r == 0 || r == H)) {
         c32 a0 = base[kx], a1 = base[kx + 1];
         c32 m0 = base[(N - kx) & (N - 1)], m1 = base[N - kx - 1];
         if (r == 0) {
@@ -174,10 +179,10 @@ __device__ __forceinline__ bool aligned16(const void* p) {
   return (reinterpret_cast<uintptr_t>(p) & 15) == 0;
 }
 
-template <int N, bool FAST_REAL, bool FAST_CPLX, int GPW>
+template <int N, bool FAST_REAL, bool FAST_CPLX, int GPW, bool PACKED>
 __global__ __launch_bounds__(64) void fft2dSmallInverse(CplxView cplx, RealView real, int padL,
                                                         int padU) {
-  using C = SmallCfg<N>;
+  using C = SmallCfg<N, PACKED>;
   constexpr int H = C::H, T = C::T, P = C::P, RS = C::RS, PS = C::PS;
   __shared__ __align__(16) c32 lds[P * PS];
 
@@ -228,8 +233,9 @@ __global__ __launch_bounds__(64) void fft2dSmallInverse(CplxView cplx, RealView 
     });
     __syncthreads();
     // pack rows 0 and H into one complex row: Q = F0 + i*FH.  At kx = 0 only the real
-    // parts are used, as in the reference (fbfft/FFT2D32.cuh:310-316).
-    {
+    // parts are used, as in the reference (fbfft/FFT2D32.cuh:310-316).  Packed
+    // operands arrive in that form.
+    if constexpr (!PACKED) {
       c32* r0 = plane + 2 * l;
       const c32* rH = r0 + H * RS;
       float4 a = ldsLoad4(r0);
@@ -240,8 +246,8 @@ __global__ __launch_bounds__(64) void fft2dSmallInverse(CplxView cplx, RealView 
         q.y = c.x;
       }
       *reinterpret_cast<float4*>(r0) = q;
+      __syncthreads();
     }
-    __syncthreads();
     rowPassInPlace<N, false>(plane, l);
     __syncthreads();
     c32 z0[H], z1[H];
@@ -338,86 +344,72 @@ bool fastCplx(int N, const CplxView& c) {
   return c.sc == 2 && c.sr == 2 * N && c.sb % 4 == 0 && aligned(c.data, 16);
 }
 
-template <int N>
+// runs f(std::bool_constant<a>{}, std::bool_constant<b>{}) for the run-time pair (a, b)
+template <typename F>
+void withFlags(bool a, bool b, F&& f) {
+  if (a && b) f(std::true_type{}, std::true_type{});
+  else if (a) f(std::true_type{}, std::false_type{});
+  else if (b) f(std::false_type{}, std::true_type{});
+  else f(std::false_type{}, std::false_type{});
+}
+
+template <int N, bool PACKED>
 int launchForward(const RealView& real, const CplxView& cplx, int padL, int padU, hipStream_t s) {
-  using C = SmallCfg<N>;
+  using C = SmallCfg<N, PACKED>;
   const int groups = ceilDiv(real.B, C::P);
-  const bool fr = fastReal(N, real, padL, padU), fc = fastCplx(N, cplx);
   dim3 block(64);
-  if (pairGroups<N>(groups)) {
-    dim3 grid(ceilDiv(groups, 2));
-    if (fr && fc)
-      fft2dSmallForward<N, true, true, 2><<<grid, block, 0, s>>>(real, cplx, padL, padU);
-    else if (fc)
-      fft2dSmallForward<N, false, true, 2><<<grid, block, 0, s>>>(real, cplx, padL, padU);
-    else if (fr)
-      fft2dSmallForward<N, true, false, 2><<<grid, block, 0, s>>>(real, cplx, padL, padU);
+  withFlags(fastReal(N, real, padL, padU), fastCplx(N, cplx), [&](auto fr, auto fc) {
+    constexpr bool FR = decltype(fr)::value, FC = decltype(fc)::value;
+    if (pairGroups<N>(groups))
+      fft2dSmallForward<N, FR, FC, 2, PACKED><<<dim3(ceilDiv(groups, 2)), block, 0, s>>>(real, cplx, padL, padU);
     else
-      fft2dSmallForward<N, false, false, 2><<<grid, block, 0, s>>>(real, cplx, padL, padU);
-  } else {
-    dim3 grid(groups);
-    if (fr && fc)
-      fft2dSmallForward<N, true, true, 1><<<grid, block, 0, s>>>(real, cplx, padL, padU);
-    else if (fc)
-      fft2dSmallForward<N, false, true, 1><<<grid, block, 0, s>>>(real, cplx, padL, padU);
-    else if (fr)
-      fft2dSmallForward<N, true, false, 1><<<grid, block, 0, s>>>(real, cplx, padL, padU);
-    else
-      fft2dSmallForward<N, false, false, 1><<<grid, block, 0, s>>>(real, cplx, padL, padU);
-  }
+      fft2dSmallForward<N, FR, FC, 1, PACKED><<<dim3(groups), block, 0, s>>>(real, cplx, padL, padU);
+  });
   return launchStatus();
 }
 
-template <int N>
+template <int N, bool PACKED>
 int launchInverse(const CplxView& cplx, const RealView& real, int padL, int padU, hipStream_t s) {
-  using C = SmallCfg<N>;
+  using C = SmallCfg<N, PACKED>;
   const int groups = ceilDiv(real.B, C::P);
-  const bool fr = fastReal(N, real, padL, padU), fc = fastCplx(N, cplx);
   dim3 block(64);
-  if (pairGroups<N>(groups)) {
-    dim3 grid(ceilDiv(groups, 2));
-    if (fr && fc)
-      fft2dSmallInverse<N, true, true, 2><<<grid, block, 0, s>>>(cplx, real, padL, padU);
-    else if (fc)
-      fft2dSmallInverse<N, false, true, 2><<<grid, block, 0, s>>>(cplx, real, padL, padU);
-    else if (fr)
-      fft2dSmallInverse<N, true, false, 2><<<grid, block, 0, s>>>(cplx, real, padL, padU);
+  withFlags(fastReal(N, real, padL, padU), fastCplx(N, cplx), [&](auto fr, auto fc) {
+    constexpr bool FR = decltype(fr)::value, FC = decltype(fc)::value;
+    if (pairGroups<N>(groups))
+      fft2dSmallInverse<N, FR, FC, 2, PACKED><<<dim3(ceilDiv(groups, 2)), block, 0, s>>>(cplx, real, padL, padU);
     else
-      fft2dSmallInverse<N, false, false, 2><<<grid, block, 0, s>>>(cplx, real, padL, padU);
-  } else {
-    dim3 grid(groups);
-    if (fr && fc)
-      fft2dSmallInverse<N, true, true, 1><<<grid, block, 0, s>>>(cplx, real, padL, padU);
-    else if (fc)
-      fft2dSmallInverse<N, false, true, 1><<<grid, block, 0, s>>>(cplx, real, padL, padU);
-    else if (fr)
-      fft2dSmallInverse<N, true, false, 1><<<grid, block, 0, s>>>(cplx, real, padL, padU);
-    else
-      fft2dSmallInverse<N, false, false, 1><<<grid, block, 0, s>>>(cplx, real, padL, padU);
-  }
+      fft2dSmallInverse<N, FR, FC, 1, PACKED><<<dim3(groups), block, 0, s>>>(cplx, real, padL, padU);
+  });
   return launchStatus();
 }
 
 }  // namespace
 
+// packed: cplx is [B][N/2][N][2] with rows 0 and N/2 of the spectrum packed in row 0
 int launchFft2dSmallForward(int N, const RealView& real, const CplxView& cplx, int padL, int padU,
-                            hipStream_t s) {
+                            hipStream_t s, bool packed) {
   if (real.B <= 0) return FBFFT_SUCCESS;
   switch (N) {
-    case 8: return launchForward<8>(real, cplx, padL, padU, s);
-    case 16: return launchForward<16>(real, cplx, padL, padU, s);
-    case 32: return launchForward<32>(real, cplx, padL, padU, s);
+    case 8: return packed ? launchForward<8, true>(real, cplx, padL, padU, s)
+                          : launchForward<8, false>(real, cplx, padL, padU, s);
+    case 16: return packed ? launchForward<16, true>(real, cplx, padL, padU, s)
+                           : launchForward<16, false>(real, cplx, padL, padU, s);
+    case 32: return packed ? launchForward<32, true>(real, cplx, padL, padU, s)
+                           : launchForward<32, false>(real, cplx, padL, padU, s);
   }
   return FBFFT_UNSUPPORTED_SIZE;
 }
 
 int launchFft2dSmallInverse(int N, const CplxView& cplx, const RealView& real, int padL, int padU,
-                            hipStream_t s) {
+                            hipStream_t s, bool packed) {
   if (real.B <= 0) return FBFFT_SUCCESS;
   switch (N) {
-    case 8: return launchInverse<8>(cplx, real, padL, padU, s);
-    case 16: return launchInverse<16>(cplx, real, padL, padU, s);
-    case 32: return launchInverse<32>(cplx, real, padL, padU, s);
+    case 8: return packed ? launchInverse<8, true>(cplx, real, padL, padU, s)
+                          : launchInverse<8, false>(cplx, real, padL, padU, s);
+    case 16: return packed ? launchInverse<16, true>(cplx, real, padL, padU, s)
+                           : launchInverse<16, false>(cplx, real, padL, padU, s);
+    case 32: return packed ? launchInverse<32, true>(cplx, real, padL, padU, s)
+                           : launchInverse<32, false>(cplx, real, padL, padU, s);
   }
   return FBFFT_UNSUPPORTED_SIZE;
 }

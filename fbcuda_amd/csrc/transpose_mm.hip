@@ -22,6 +22,18 @@
 // Cim = k1 + k2).  C leaves through LDS
 // so that stores cover whole runs.  Only this contraction uses MFMA; it is the
 // one dense product of the convolution path.
+//
+// Packed spectra (fbfft_transpose_mm_packed): operands [..][..][N/2][N] whose row 0
+// holds P[x] = F0[x] + i FH[x], the spectra of the two real rows 0 and N/2 of an
+// N x N transform (the Unpack = false format of fbfft/FFT2D32.cuh:421-427).  Rows
+// 1 .. N/2-1 are plain bins and go through the kernel above.  Row 0 follows the
+// product rule of fbfft/FFTIteratedConvolution.cuh:161-186: unpack both operands,
+// multiply F0 with F0 and FH with FH, re-pack.  The PACKED0 variant of the kernel
+// does that on the way into and out of LDS: a workgroup takes four x (0 < x < N/2)
+// and its eight waves own the "virtual bins" F0[x] and FH[x], computed from P[x] and
+// P[N-x] when a slice is parked; the epilogue combines C0[x] and CH[x] into P[x] and
+// P[N-x].  x = 0 pairs with x = N/2: both hold two real values, which multiply
+// component by component (no cross terms).
 #include "common.h"
 
 namespace fbfft_amd {
@@ -64,12 +76,33 @@ struct Fetch {
 // values outside it are zeroed only when the slice is parked in LDS one iteration
 // later, so nothing waits for a load between its issue and the products of the
 // current slice.  VEC4 additionally needs XY even (a bin pair never straddles the end).
-template <bool VEC4>
+// bin that shares its two spectra with bin x of a packed row 0
+__device__ __forceinline__ int packedPartner(int x, int N) { return x == 0 ? N / 2 : N - x; }
+
+// PACKED0: XY is the length N of packed row 0, x0 a multiple of 4 below N/2; lane
+// t fetches P[x] and P[partner(x)] for x = x0 + t % 4.
+template <bool VEC4, bool PACKED0>
 __device__ __forceinline__ Fetch fetchSlice(const float* base, long rowStride, long kStride,
                                             int rows, int row0, int K, int k0, int XY, int x0,
                                             int t) {
   Fetch f;
   const int p = t % 4;
+  if constexpr (PACKED0) {
+    const int e = t / 4;
+    const int row = row0 + e % 64;
+    const int x = x0 + p;
+    const float* src0 = base + (long)min(row, rows - 1) * rowStride;
+    const long o1 = 2L * x, o2 = 2L * packedPartner(x, XY);
+#pragma unroll
+    for (int u = 0; u < KC / 2; ++u) {
+      const int k = k0 + e / 64 + 2 * u;
+      const float* src = src0 + (long)min(k, K - 1) * kStride;
+      const float2 a = *reinterpret_cast<const float2*>(src + o1);
+      const float2 b = *reinterpret_cast<const float2*>(src + o2);
+      f.v[u] = float4{a.x, a.y, b.x, b.y};
+    }
+    return f;
+  }
   const int x = x0 + 2 * p;
   const int e = t / 4;
   const int row = row0 + e % 64;
@@ -92,11 +125,33 @@ __device__ __forceinline__ Fetch fetchSlice(const float* base, long rowStride, l
 
 // Parks a fetched slice (k0 .. k0 + KC) in its LDS planes, zeroing what lies outside
 // the operand.
+template <bool PACKED0>
 __device__ __forceinline__ void stashSlice(float* re, float* im, const Fetch& f, float sign,
                                            int rows, int row0, int K, int k0, int XY, int x0,
                                            int t) {
   const int p = t % 4;
   const int e = t / 4;
+  if constexpr (PACKED0) {
+    // virtual bin p: F0[x], virtual bin 4 + p: FH[x]; for x = 0 the two bins hold the
+    // real pairs (F0[0], F0[N/2]) and (FH[0], FH[N/2]), which conjugation leaves alone
+    const bool ok0 = row0 + e % 64 < rows;
+    const bool ends = x0 + p == 0;
+#pragma unroll
+    for (int u = 0; u < KC / 2; ++u) {
+      const int o = (e / 64 + 2 * u) * 64 + e % 64;
+      const bool ok = ok0 && k0 + e / 64 + 2 * u < K;
+      const float4 v = f.v[u];  // P[x] = (v.x, v.y), P[partner] = (v.z, v.w)
+      const float r0 = ends ? v.x : 0.5f * (v.x + v.z);
+      const float i0 = ends ? v.z : sign * 0.5f * (v.y - v.w);
+      const float rH = ends ? v.y : 0.5f * (v.y + v.w);
+      const float iH = ends ? v.w : sign * 0.5f * (v.z - v.x);
+      re[p * XS + o] = ok ? r0 : 0.f;
+      im[p * XS + o] = ok ? i0 : 0.f;
+      re[(4 + p) * XS + o] = ok ? rH : 0.f;
+      im[(4 + p) * XS + o] = ok ? iH : 0.f;
+    }
+    return;
+  }
   const int x = x0 + 2 * p;
   const bool ok0 = row0 + e % 64 < rows && x < XY;
   const bool okX1 = x + 1 < XY;
@@ -111,7 +166,7 @@ __device__ __forceinline__ void stashSlice(float* re, float* im, const Fetch& f,
   }
 }
 
-template <bool VEC4>
+template <bool VEC4, bool PACKED0>
 __global__ __launch_bounds__(THREADS) void transposeMMKernel(MMArgs a) {
   __shared__ __align__(8) float lds[LDS_FLOATS];  // two slice buffers; later the C staging area
   const int t = threadIdx.x;
@@ -125,8 +180,11 @@ __global__ __launch_bounds__(THREADS) void transposeMMKernel(MMArgs a) {
   const int per = (total + 7) / 8;
   const int logical = (blockIdx.x % 8) * per + blockIdx.x / 8;
   if (logical >= total) return;
-  const int x0 = (logical / (tilesI * tilesJ)) * XB;
+  const int x0 = (logical / (tilesI * tilesJ)) * (PACKED0 ? XB / 2 : XB);
   const int rem = logical % (tilesI * tilesJ);
+  // PACKED0: the waves holding the real pairs of x = 0 multiply component by component
+  const bool ends = PACKED0 && x0 == 0 && w % 4 == 0;
+  const float cross = ends ? 0.f : 1.f;
   const int j0 = (rem % tilesJ) * TJ;
   const int i0 = (rem / tilesJ) * TI;
 
@@ -148,13 +206,14 @@ __global__ __launch_bounds__(THREADS) void transposeMMKernel(MMArgs a) {
 
   Fetch fa, fb;
   auto fetchAll = [&](int k0) __attribute__((always_inline)) {
-    fa = fetchSlice<VEC4>(a.A, a.aRow, a.aK, a.I, i0, a.K, k0, a.XY, x0, t);
-    fb = fetchSlice<VEC4>(a.B, a.bCol, a.bK, a.J, j0, a.K, k0, a.XY, x0, t);
+    fa = fetchSlice<VEC4, PACKED0>(a.A, a.aRow, a.aK, a.I, i0, a.K, k0, a.XY, x0, t);
+    fb = fetchSlice<VEC4, PACKED0>(a.B, a.bCol, a.bK, a.J, j0, a.K, k0, a.XY, x0, t);
   };
   auto stashAll = [&](int buf, int k0) __attribute__((always_inline)) {
     float* base = lds + buf * BUF;
-    stashSlice(base, base + PLANE, fa, a.aSign, a.I, i0, a.K, k0, a.XY, x0, t);
-    stashSlice(base + 2 * PLANE, base + 3 * PLANE, fb, a.bSign, a.J, j0, a.K, k0, a.XY, x0, t);
+    stashSlice<PACKED0>(base, base + PLANE, fa, a.aSign, a.I, i0, a.K, k0, a.XY, x0, t);
+    stashSlice<PACKED0>(base + 2 * PLANE, base + 3 * PLANE, fb, a.bSign, a.J, j0, a.K, k0, a.XY,
+                        x0, t);
   };
   // Two slice buffers, one barrier per slice: while the waves multiply slice n out
   // of one buffer, each of them first parks slice n+1 (already in its registers) in
@@ -191,9 +250,15 @@ __global__ __launch_bounds__(THREADS) void transposeMMKernel(MMArgs a) {
       float as[2], bd[2], bs[2];
 #pragma unroll
       for (int q = 0; q < 2; ++q) {
-        as[q] = ar[q] + ai[q];
+        if constexpr (PACKED0) {
+          // real pairs: k1 = sum ar br and k3 = sum ai bi are the two results
+          as[q] = __builtin_fmaf(cross, ai[q], ar[q]);
+          bs[q] = __builtin_fmaf(cross, br[q], bi[q]);
+        } else {
+          as[q] = ar[q] + ai[q];
+          bs[q] = br[q] + bi[q];
+        }
         bd[q] = bi[q] - br[q];
-        bs[q] = br[q] + bi[q];
       }
 #pragma unroll
       for (int si = 0; si < 2; ++si)
@@ -222,9 +287,12 @@ __global__ __launch_bounds__(THREADS) void transposeMMKernel(MMArgs a) {
       for (int sj = 0; sj < 2; ++sj)
 #pragma unroll
         for (int rr = 0; rr < 4; ++rr)
+        {
+          const float v1 = k1[si][sj][4 * c + rr], v2 = k2[si][sj][4 * c + rr],
+                      v3 = k3[si][sj][4 * c + rr];
           stage[((4 * hh + rr) * TJ + 32 * sj + col) * CSTR + w] =
-              float2{k1[si][sj][4 * c + rr] - k3[si][sj][4 * c + rr],
-                     k1[si][sj][4 * c + rr] + k2[si][sj][4 * c + rr]};
+              ends ? float2{v1, v3} : float2{v1 - v3, v1 + v2};
+        }
       __syncthreads();
       // 512 (row, col) elements x 8 bins: 8 lanes per element, 64 elements per pass
       const int xl = t % 8;
@@ -232,9 +300,25 @@ __global__ __launch_bounds__(THREADS) void transposeMMKernel(MMArgs a) {
       for (int pass = 0; pass < 8; ++pass) {
         const int e = t / 8 + 64 * pass;  // 0..511
         const int row = e / TJ, cc = e % TJ;
-        const int i = i0 + 32 * si + 8 * c + row, j = j0 + cc, x = x0 + xl;
+        const int i = i0 + 32 * si + 8 * c + row, j = j0 + cc;
+        int x = x0 + xl;
+        float2 acc;
+        if constexpr (PACKED0) {
+          // lanes 0..3: P[x], lanes 4..7: P[partner(x)], from C0[x] and CH[x]
+          const int q = xl % 4;
+          const bool second = xl >= 4;
+          const float2 c0 = stage[(row * TJ + cc) * CSTR + q];
+          const float2 cH = stage[(row * TJ + cc) * CSTR + 4 + q];
+          x = x0 + q;
+          if (x == 0)
+            acc = second ? float2{c0.y, cH.y} : float2{c0.x, cH.x};
+          else
+            acc = second ? float2{c0.x + cH.y, cH.x - c0.y} : float2{c0.x - cH.y, c0.y + cH.x};
+          if (second) x = packedPartner(x, a.XY);
+        } else {
+          acc = stage[(row * TJ + cc) * CSTR + xl];
+        }
         if (i < a.I && j < a.J && x < a.XY) {
-          float2 acc = stage[(row * TJ + cc) * CSTR + xl];
           float* dst = a.C + (long)i * a.cRow + (long)j * a.cCol + 2L * x;
           if (a.accumulate) {
             float2 old = *reinterpret_cast<const float2*>(dst);
@@ -280,9 +364,44 @@ int launchTransposeMM(const float* A, long a0, long a1, const float* B, long b0,
   const bool vec4 = aligned(A, 16) && aligned(B, 16) && a0 % 4 == 0 && a1 % 4 == 0 &&
                     b0 % 4 == 0 && b1 % 4 == 0 && XY % 2 == 0;
   if (vec4)
-    transposeMMKernel<true><<<grid, block, 0, s>>>(m);
+    transposeMMKernel<true, false><<<grid, block, 0, s>>>(m);
   else
-    transposeMMKernel<false><<<grid, block, 0, s>>>(m);
+    transposeMMKernel<false, false><<<grid, block, 0, s>>>(m);
+  return launchStatus();
+}
+
+// The same contraction on packed spectra [d0][d1][N/2][N][2]: rows 1 .. N/2-1 as
+// plain bins, row 0 by the unpack / multiply / re-pack rule.
+int launchTransposeMMPacked(const float* A, long a0, long a1, const float* B, long b0, long b1,
+                            float* C, long c0, long c1, int I, int J, int K, int N, bool conjA,
+                            bool conjB, bool accumulate, float invNorm, hipStream_t s) {
+  if (I <= 0 || J <= 0) return FBFFT_SUCCESS;
+  if (N > 2) {
+    const int rc = launchTransposeMM(A + 2 * N, a0, a1, B + 2 * N, b0, b1, C + 2 * N, c0, c1, I, J,
+                                     K, (N / 2 - 1) * N, conjA, conjB, accumulate, invNorm, s);
+    if (rc != FBFFT_SUCCESS) return rc;
+  }
+  MMArgs m;
+  m.A = A;
+  m.B = B;
+  m.C = C;
+  m.I = I;
+  m.J = J;
+  m.K = K;
+  m.XY = N;
+  m.aRow = conjA ? a1 : a0;
+  m.aK = conjA ? a0 : a1;
+  m.bK = conjB ? b1 : b0;
+  m.bCol = conjB ? b0 : b1;
+  m.cRow = c0;
+  m.cCol = c1;
+  m.aSign = conjA ? -1.f : 1.f;
+  m.bSign = conjB ? -1.f : 1.f;
+  m.invNorm = invNorm;
+  m.accumulate = accumulate ? 1 : 0;
+  m.chunks = N / XB;  // four x per workgroup, x < N/2
+  const int total = m.chunks * ceilDiv(J, TJ) * ceilDiv(I, TI);
+  transposeMMKernel<false, true><<<dim3((total + 7) / 8 * 8), dim3(THREADS), 0, s>>>(m);
   return launchStatus();
 }
 

@@ -83,7 +83,10 @@ int fbfft_c2r_1d(const fbfft_tensor* real, const fbfft_tensor* cplx, int padL,
  *   cplx [B][N/2+1][N][2], N in {64,128}:   cplx[b][kx][ky]  (one kernel; an
  *       extension: the reference needs two calls and a scratch buffer)
  *   cplx [B][N][N/2+1][2], N in {64,128}:   the reference's first pass: row
- *       transforms into the caller's scratch, cplx[b][y][kx]. */
+ *       transforms into the caller's scratch, cplx[b][y][kx].
+ *   cplx [B][N/2][N][2],   N in {8,16,32}:  the packed format (Unpack = false,
+ *       fbfft/FFT2D32.cuh:421-427): rows 1 .. N/2-1 as above, row 0 holds
+ *       F[0][kx] + i F[N/2][kx] (both spectra are those of real rows). */
 int fbfft_r2c_2d(const fbfft_tensor* real, const fbfft_tensor* cplx, int padL, int padU,
                  fbfft_stream_t stream);
 
@@ -98,7 +101,9 @@ int fbfft_c2c_2d_pass2(const fbfft_tensor* src, const fbfft_tensor* dst, fbfft_s
  *   cplx [B][N/2+1][N][2], N in {8,16,32}:  one kernel
  *   cplx [B][N/2+1][N][2], N in {64,128}:   one kernel (extension, as above)
  *   cplx [B][N][N][2],     N in {64,128}:   the reference's second inverse pass
- *       over the scratch produced by fbfft_c2c_2d_inverse_pass1. */
+ *       over the scratch produced by fbfft_c2c_2d_inverse_pass1.
+ *   cplx [B][N/2][N][2],   N in {8,16,32}:  packed input (PackedInput = true,
+ *       fbfft/FFT2D32.cuh:302-316). */
 int fbfft_c2r_2d(const fbfft_tensor* cplx, const fbfft_tensor* real, int padL, int padU,
                  fbfft_stream_t stream);
 
@@ -121,6 +126,21 @@ int fbfft_c2c_2d_inverse_pass1(const fbfft_tensor* src, const fbfft_tensor* dst,
 int fbfft_transpose_mm(const fbfft_tensor* A, const fbfft_tensor* B, const fbfft_tensor* C,
                        int conjA, int conjB, int accumulate, float invNorm,
                        fbfft_stream_t stream);
+
+/* The same contraction on PACKED spectra: A, B, C are rank-5 tensors
+ * [d0][d1][N/2][N][2], N in {8,16,32}, as fbfft_r2c_2d stores them when cplx has
+ * N/2 rows (the Unpack = false format of fbfft/FFT2D32.cuh:421-427): rows
+ * 1 .. N/2-1 are plain bins; row 0 holds P[x] = F[0][x] + i F[N/2][x] and follows
+ * the product rule of the fused kernels (fbfft/FFTIteratedConvolution.cuh:161-186,
+ * :485-504): both operands are unpacked, rows 0 and N/2 are multiplied
+ * separately, and the result is packed again, so that C can go straight into
+ * fbfft_c2r_2d in its packed form (fbfft2DVerticalCoreInverse<N, true>,
+ * fbfft/FFT2D32.cuh:302-316).  The reference declares the format but ships no
+ * contraction for it ("If a specialized gemm kernel is available, no need to
+ * unpack", FFT2D32.cuh:422). */
+int fbfft_transpose_mm_packed(const fbfft_tensor* A, const fbfft_tensor* B, const fbfft_tensor* C,
+                              int conjA, int conjB, int accumulate, float invNorm,
+                              fbfft_stream_t stream);
 
 /* detail::FFTIteratedConvolution<FFTSize> (fbfft/FFTIteratedConvolution.cuh:624-755).
  * ins / outs are DEVICE pointers to numTiles descriptors each.  weight is

@@ -3,8 +3,8 @@
 // fbcuda's fbfft headers compiles unchanged apart from the stream type
 // (hipStream_t instead of cudaStream_t).  Header-only; link libfbfft_amd.so.
 //
-//   facebook::cuda::DeviceTensor<T, Dim>                  DeviceTensor.cuh:53-246 (host-side view only)
-//   facebook::cuda::Complex                               Complex.cuh:16-140 (storage only)
+//   facebook::cuda::DeviceTensor<T, Dim>                  DeviceTensor.cuh:53-246 (the host-side interface)
+//   facebook::cuda::Complex                               Complex.cuh:16-140
 //   facebook::cuda::fbfft::FBFFTParameters                fbfft/FBFFTParameters.h:7-59
 //   facebook::cuda::fbfft::fbfft1D / fbifft1D / fbfft2D / fbifft2D   fbfft/FBFFT.cuh:11-56
 //   facebook::cuda::transposeMM                           MM.cuh:11-17
@@ -13,13 +13,21 @@
 #ifndef FBFFT_AMD_HPP
 #define FBFFT_AMD_HPP
 
+#include <cmath>
 #include <cstddef>
+#include <stdexcept>
+#include <string>
+#include <utility>
+#include <vector>
 
 #include "fbfft_amd.h"
 
 namespace facebook { namespace cuda {
 
-// Two packed floats, layout-compatible with the reference's cuComplex wrapper.
+// Two packed floats, layout-compatible with the reference's cuComplex wrapper
+// (Complex.cuh:16-140), with its host-side arithmetic: products and quotients follow
+// cuComplex.h (cuCmulf: (ac - bd, ad + bc); cuCdivf: both operands scaled by
+// 1 / (|c| + |d|) before the division).
 struct Complex {
   float re_, im_;
   Complex() : re_(0.f), im_(0.f) {}
@@ -31,17 +39,68 @@ struct Complex {
   const float& im() const { return im_; }
   Complex conjugate() const { return Complex(re_, -im_); }
   Complex transpose() const { return Complex(im_, re_); }
+  void cexp(float angle) { re_ = std::cos(angle); im_ = std::sin(angle); }
+
+  bool operator==(const Complex& o) const { return re_ == o.re_ && im_ == o.im_; }
+  bool operator!=(const Complex& o) const { return !(*this == o); }
+  Complex operator-() const { return Complex(-re_, -im_); }
+  Complex operator+(const Complex& o) const { return Complex(re_ + o.re_, im_ + o.im_); }
+  Complex operator-(const Complex& o) const { return Complex(re_ - o.re_, im_ - o.im_); }
+  Complex operator*(const Complex& o) const {
+    return Complex(re_ * o.re_ - im_ * o.im_, re_ * o.im_ + im_ * o.re_);
+  }
+  Complex operator/(const Complex& o) const {
+    const float scale = 1.0f / (std::fabs(o.re_) + std::fabs(o.im_));
+    const float ar = re_ * scale, ai = im_ * scale, br = o.re_ * scale, bi = o.im_ * scale;
+    const float inv = 1.0f / (br * br + bi * bi);
+    return Complex((ar * br + ai * bi) * inv, (ai * br - ar * bi) * inv);
+  }
+  Complex& operator+=(const Complex& o) { return *this = *this + o; }
+  Complex& operator-=(const Complex& o) { return *this = *this - o; }
+  Complex& operator*=(const Complex& o) { return *this = *this * o; }
+  Complex& operator/=(const Complex& o) { return *this = *this / o; }
 };
 static_assert(sizeof(Complex) == 8, "Complex is two packed floats");
 
+template <typename T, int Dim, typename IndexT>
+class DeviceTensor;
+
+namespace fbfft_amd_detail {
+
+// tensor[i][j]...: the address arithmetic of the reference's DeviceSubTensor
+// (DeviceTensor.cuh:249-379) for host code, which can only take addresses of
+// device memory: data() of the indexed element or sub-tensor.
+template <typename T, int Left, typename IndexT>
+class SubView {
+ public:
+  SubView(T* at, const IndexT* strides) : at_(at), strides_(strides) {}
+  SubView<T, Left - 1, IndexT> operator[](IndexT i) const {
+    static_assert(Left >= 1, "too many indices");
+    return SubView<T, Left - 1, IndexT>(at_ + (std::ptrdiff_t)i * strides_[0], strides_ + 1);
+  }
+  T* data() const { return at_; }
+
+ private:
+  T* at_;
+  const IndexT* strides_;
+};
+
+}  // namespace fbfft_amd_detail
+
 // Non-owning strided view with the reference's member order (data, strides,
-// sizes); strides count elements of T.  Only what host code needs to describe an
-// operand is provided: the kernels receive plain pointers and ints.
+// sizes) and its host-side interface (DeviceTensor.cuh:53-246,
+// DeviceTensor-inl.cuh); strides count elements of T.  Everything here is size /
+// stride arithmetic on the host: the kernels receive plain pointers and ints.
+// Invariant violations throw std::invalid_argument, as the reference's host code does.
 template <typename T, int Dim, typename IndexT = int>
 class DeviceTensor {
  public:
   enum { NumDim = Dim };
   typedef T DataType;
+  typedef IndexT IndexType;
+  typedef T* DataPtrType;
+  typedef DeviceTensor<T, Dim, IndexT> TensorType;
+  static_assert(Dim > 0, "rank");
 
   DeviceTensor() : data_(nullptr) {
     for (int i = 0; i < Dim; ++i) { stride_[i] = 0; size_[i] = 0; }
@@ -59,10 +118,163 @@ class DeviceTensor {
   T* data() { return data_; }
   const T* data() const { return data_; }
   template <typename U> U* dataAs() { return reinterpret_cast<U*>(data_); }
+  template <typename U> const U* dataAs() const { return reinterpret_cast<const U*>(data_); }
   IndexT getSize(int i) const { return size_[i]; }
   IndexT getStride(int i) const { return stride_[i]; }
   const IndexT* sizes() const { return size_; }
   const IndexT* strides() const { return stride_; }
+
+  fbfft_amd_detail::SubView<T, Dim - 1, IndexT> operator[](IndexT i) const {
+    return fbfft_amd_detail::SubView<T, Dim - 1, IndexT>(data_ + (std::ptrdiff_t)i * stride_[0],
+                                                         stride_ + 1);
+  }
+
+  template <int OtherDim>
+  bool isSameSize(const DeviceTensor<T, OtherDim, IndexT>& rhs) const {
+    if (Dim != OtherDim) return false;
+    for (int i = 0; i < Dim; ++i)
+      if (size_[i] != rhs.getSize(i)) return false;
+    return true;
+  }
+  template <int OtherDim>
+  bool isSameSizeAndStride(const DeviceTensor<T, OtherDim, IndexT>& rhs) const {
+    if (!isSameSize(rhs)) return false;
+    for (int i = 0; i < Dim; ++i)
+      if (stride_[i] != rhs.getStride(i)) return false;
+    return true;
+  }
+
+  // "sizes: [a, b]  strides: [c, d]"
+  std::string toString() const {
+    auto list = [](const IndexT* v) {
+      std::string out = "[";
+      for (int i = 0; i < Dim; ++i) out += (i ? ", " : "") + std::to_string(v[i]);
+      return out + "]";
+    };
+    return "sizes: " + list(size_) + "  strides: " + list(stride_);
+  }
+
+  // the same view on elements of another type of the same width
+  template <typename U>
+  DeviceTensor<U, Dim, IndexT> cast() const {
+    static_assert(sizeof(U) == sizeof(T), "cast keeps the element width");
+    return DeviceTensor<U, Dim, IndexT>(reinterpret_cast<U*>(data_), size_, stride_);
+  }
+
+  long numElements() const {
+    long n = 1;
+    for (int i = 0; i < Dim; ++i) n *= size_[i];
+    return n;
+  }
+
+  // dimension i directly encloses dimension i + 1 (no padding between them)
+  bool isContiguousDim(int i) const {
+    if (i == Dim - 1) return true;
+    return i >= 0 && i < Dim - 1 && stride_[i] / stride_[i + 1] == size_[i + 1];
+  }
+  // dense row-major, dimensions of size 1 aside
+  bool isContiguous() const {
+    long expect = 1;
+    for (int i = Dim - 1; i >= 0; --i) {
+      if (size_[i] == 1) continue;
+      if (stride_[i] != expect) return false;
+      expect *= size_[i];
+    }
+    return true;
+  }
+  // stride positive and, for i > 0, no larger extent than the enclosing stride allows
+  bool isConsistentlySized(int i) const {
+    if (i < 0 || i >= Dim || stride_[i] <= 0) return false;
+    return i == 0 ? size_[0] > 0 : stride_[i - 1] / stride_[i] >= size_[i];
+  }
+  bool isConsistentlySized() const {
+    for (int i = 0; i < Dim; ++i)
+      if (!isConsistentlySized(i)) return false;
+    return true;
+  }
+
+  // Reorders the SIZES by perm and recomputes dense strides (the data is not moved);
+  // dense tensors only.
+  void permuteDims(const std::vector<int>& perm) {
+    if ((int)perm.size() != Dim)
+      throw std::invalid_argument("Permutation list must be of the same size as our dimension");
+    if (stride_[Dim - 1] != 1) throw std::invalid_argument("Innermost dimension must have stride 1");
+    for (int i = 0; i < Dim; ++i)
+      if (!isContiguousDim(i)) throw std::invalid_argument("All dimensions must be contiguous");
+    IndexT sz[Dim];
+    for (int i = 0; i < Dim; ++i) sz[i] = size_[perm[i]];
+    *this = DeviceTensor(data_, sz);
+  }
+
+  // sizes and strides of two dimensions exchanged; no data movement
+  DeviceTensor transpose(int dim1, int dim2) const {
+    if (dim1 < 0 || dim1 >= Dim) throw std::invalid_argument("dim1 out of bounds");
+    if (dim2 < 0 || dim2 >= Dim) throw std::invalid_argument("dim2 out of bounds");
+    DeviceTensor t = *this;
+    std::swap(t.size_[dim1], t.size_[dim2]);
+    std::swap(t.stride_[dim1], t.stride_[dim2]);
+    return t;
+  }
+
+  // [2][3] -> [1][1][2][3]; the new dimensions stride over the whole tensor
+  template <int NewDim>
+  DeviceTensor<T, NewDim, IndexT> upcastOuter() const {
+    static_assert(NewDim > Dim, "upcast raises the rank");
+    IndexT sz[NewDim], st[NewDim];
+    for (int i = 0; i < NewDim - Dim; ++i) { sz[i] = 1; st[i] = size_[0] * stride_[0]; }
+    for (int i = 0; i < Dim; ++i) { sz[NewDim - Dim + i] = size_[i]; st[NewDim - Dim + i] = stride_[i]; }
+    return DeviceTensor<T, NewDim, IndexT>(data_, sz, st);
+  }
+  // [2][3] -> [2][3][1][1]
+  template <int NewDim>
+  DeviceTensor<T, NewDim, IndexT> upcastInner() const {
+    static_assert(NewDim > Dim, "upcast raises the rank");
+    IndexT sz[NewDim], st[NewDim];
+    for (int i = 0; i < NewDim; ++i) { sz[i] = i < Dim ? size_[i] : 1; st[i] = i < Dim ? stride_[i] : 1; }
+    return DeviceTensor<T, NewDim, IndexT>(data_, sz, st);
+  }
+  // [a][b][c][d] -> [a*b*c][d] for NewDim = 2: the leading dimensions collapse into
+  // the first one kept; they must enclose each other without padding
+  template <int NewDim>
+  DeviceTensor<T, NewDim, IndexT> downcastOuter() const {
+    static_assert(NewDim < Dim, "downcast lowers the rank");
+    constexpr int gone = Dim - NewDim;
+    IndexT sz[NewDim], st[NewDim];
+    IndexT lead = 1;
+    for (int i = 0; i < gone; ++i) {
+      if (!isContiguousDim(i)) throw std::invalid_argument("Can only downcast contiguous tensors");
+      lead *= size_[i];
+    }
+    for (int i = 0; i < NewDim; ++i) { sz[i] = size_[gone + i]; st[i] = stride_[gone + i]; }
+    sz[0] *= lead;
+    return DeviceTensor<T, NewDim, IndexT>(data_, sz, st);
+  }
+  // [a][b][c][d] -> [a][b*c*d] for NewDim = 2: the trailing dimensions collapse into
+  // the last one kept, which takes the innermost stride
+  template <int NewDim>
+  DeviceTensor<T, NewDim, IndexT> downcastInner() const {
+    static_assert(NewDim < Dim, "downcast lowers the rank");
+    IndexT sz[NewDim], st[NewDim];
+    IndexT tail = 1;
+    for (int i = NewDim; i < Dim; ++i) {
+      if (!isContiguousDim(i)) throw std::invalid_argument("Can only downcast contiguous tensors");
+      tail *= size_[i];
+    }
+    for (int i = 0; i < NewDim; ++i) { sz[i] = size_[i]; st[i] = stride_[i]; }
+    sz[NewDim - 1] *= tail;
+    st[NewDim - 1] = stride_[Dim - 1];
+    return DeviceTensor<T, NewDim, IndexT>(data_, sz, st);
+  }
+  // the innermost SubDim dimensions as a tensor starting at `at`
+  template <int SubDim>
+  DeviceTensor<T, SubDim, IndexT> view(T* at) const {
+    static_assert(SubDim >= 1 && SubDim < Dim, "a view has lower rank");
+    return DeviceTensor<T, SubDim, IndexT>(at, size_ + (Dim - SubDim), stride_ + (Dim - SubDim));
+  }
+  template <int SubDim>
+  DeviceTensor<T, SubDim, IndexT> view() const {
+    return view<SubDim>(data_);
+  }
 
  private:
   T* data_;
@@ -278,6 +490,19 @@ void transposeMM(DeviceTensor<float, Dim>& A, DeviceTensor<float, Dim>& B,
   fbfft_tensor a = fbfft_amd_detail::describe(A), b = fbfft_amd_detail::describe(B),
                c = fbfft_amd_detail::describe(C);
   fbfft_transpose_mm(&a, &b, &c, ConjugateTransposeA, ConjugateTransposeB, Accumulate, invNorm, s);
+}
+
+// transposeMM on spectra in the packed format of fbfft2D (DeviceTensor<float, 5>
+// [d0][d1][N/2][N][2], N in {8,16,32}; fbfft/FFT2D32.cuh:421-427 declares the
+// format, the reference ships no contraction for it): see fbfft_transpose_mm_packed.
+template <bool ConjugateTransposeA, bool ConjugateTransposeB, bool Accumulate>
+fbfft::FBFFTParameters::ErrorCode transposeMMPacked(DeviceTensor<float, 5>& A, DeviceTensor<float, 5>& B,
+                                             DeviceTensor<float, 5>& C, float invNorm,
+                                             fbfft_stream_t s = 0) {
+  fbfft_tensor a = fbfft_amd_detail::describe(A), b = fbfft_amd_detail::describe(B),
+               c = fbfft_amd_detail::describe(C);
+  return (fbfft::FBFFTParameters::ErrorCode)fbfft_transpose_mm_packed(
+      &a, &b, &c, ConjugateTransposeA, ConjugateTransposeB, Accumulate, invNorm, s);
 }
 
 // The three passes of a convolution layer on the split FFT -> transposeMM -> IFFT

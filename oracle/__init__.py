@@ -105,6 +105,41 @@ def fbifft2d(cplx, h, w, padL=0, padU=0, out=None):
     return rc, out
 
 
+def fbfft2d_packed(real, N, padL=0, padU=0):
+    """Packed spectrum format [B][N/2][N][2] (Unpack = false, FFT2D32.cuh:421-427)."""
+    real = _f32(real)
+    B, h, w = real.shape
+    out = np.zeros((B, N // 2, N, 2), np.float32)
+    rc = lib().orc_fbfft2d_packed(_p(real), B, h, w, N, padL, padU, _p(out))
+    return rc, out
+
+
+def fbifft2d_packed(cplx, h, w, padL=0, padU=0):
+    cplx = _f32(cplx)
+    B, nr, N, _ = cplx.shape
+    assert nr == N // 2
+    out = np.zeros((B, h, w), np.float32)
+    rc = lib().orc_fbifft2d_packed(_p(cplx), B, N, h, w, padL, padU, _p(out))
+    return rc, out
+
+
+def transpose_mm_packed(A, B, conjA, conjB, invNorm, C=None):
+    """A, B packed spectra [..][..][N/2][N][2]; returns C [I][J][N/2][N][2]."""
+    A, B = _f32(A), _f32(B)
+    N = A.shape[3]
+    assert A.shape[2] == N // 2 and B.shape[2:] == A.shape[2:]
+    if conjA:
+        K, I = A.shape[:2]
+    else:
+        I, K = A.shape[:2]
+    J = B.shape[0] if conjB else B.shape[1]
+    accumulate = C is not None
+    C = np.zeros((I, J, N // 2, N, 2), np.float32) if C is None else _f32(C).copy()
+    lib().orc_transpose_mm_packed(_p(A), _p(B), _p(C), I, J, K, N, int(conjA), int(conjB),
+                                  int(accumulate), ctypes.c_float(invNorm))
+    return C
+
+
 def transpose_mm(A, B, conjA, conjB, invNorm, C=None):
     """A, B complex-as-float [..][..][XY][2]; returns C [I][J][XY][2]."""
     A, B = _f32(A), _f32(B)

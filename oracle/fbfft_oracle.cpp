@@ -295,24 +295,31 @@ inline void unpackRow0(const cf* a, int N, int x, cf* r0, cf* rN2) {
   }
 }
 
+// packed: the Unpack = false store (FFT2D32.cuh:421-427), out is [N/2][N]
 void fbfft2dSmallPlane(const float* plane, int h, int w, int N, int padL, int padU,
-                       float* out) {
+                       float* out, bool packed = false) {
   const int H = N / 2;
   std::vector<cf> a((size_t)H * N);
   loadPacked(a.data(), N, plane, h, w, w, padL, padU);
   coreForward(a.data(), N);
   cf* o = reinterpret_cast<cf*>(out);  // [N/2+1][N]
+  if (packed) {
+    for (int i = 0; i < H; ++i)
+      for (int x = 0; x < N; ++x) o[i * N + x] = a[i * N + x];
+    return;
+  }
   for (int i = 1; i < H; ++i)
     for (int x = 0; x < N; ++x) o[i * N + x] = a[i * N + x];
   for (int x = 0; x < N; ++x) unpackRow0(a.data(), N, x, &o[x], &o[H * N + x]);
 }
 
+// packed: PackedInput = true (FFT2D32.cuh:446-458), in is [N/2][N]
 void fbifft2dSmallPlane(const float* in, int N, int h, int w, int padL, int padU,
-                        float* plane) {
+                        float* plane, bool packed = false) {
   const int H = N / 2;
   std::vector<cf> a((size_t)(H + 1) * N);
-  std::memcpy(a.data(), in, sizeof(cf) * (size_t)(H + 1) * N);
-  coreInverse(a.data(), N, false);
+  std::memcpy(a.data(), in, sizeof(cf) * (size_t)(packed ? H : H + 1) * N);
+  coreInverse(a.data(), N, packed);
   // FFT2D32.cuh:462-469
   for (int i = 0; i < N; i += 2) {
     for (int x = 0; x < N; ++x) {
@@ -567,6 +574,82 @@ int orc_fbifft2d(const float* cplx, int B, int N, int h, int w, int padL, int pa
     }
   }
   return 0;
+}
+
+// fbfft2DVertical<..., Unpack = false> (FFT2D32.cuh:361-427): real [B][h][w] ->
+// cplx [B][N/2][N][2], N in {8,16,32}; row 0 holds F[0][kx] + i F[N/2][kx].  The
+// reference declares this store but instantiates no kernel with it
+// (FFT2D32.cuh:473-502 use the default); the fused convolution kernels consume the
+// same in-register form.
+int orc_fbfft2d_packed(const float* real, int B, int h, int w, int N, int padL, int padU,
+                       float* cplx) {
+  if (!(N == 8 || N == 16 || N == 32)) return 1;
+  const size_t inPlane = (size_t)h * w, outPlane = (size_t)(N / 2) * N * 2;
+#pragma omp parallel for schedule(static)
+  for (int b = 0; b < B; ++b)
+    fbfft2dSmallPlane(real + b * inPlane, h, w, N, padL, padU, cplx + b * outPlane, true);
+  return 0;
+}
+
+// fbifft2DVertical<..., PackedInput = true> (FFT2D32.cuh:430-470, core :302-358):
+// cplx [B][N/2][N][2] -> real [B][h][w], gain N*N.
+int orc_fbifft2d_packed(const float* cplx, int B, int N, int h, int w, int padL, int padU,
+                        float* real) {
+  if (!(N == 8 || N == 16 || N == 32)) return 1;
+  const size_t outPlane = (size_t)h * w, inPlane = (size_t)(N / 2) * N * 2;
+#pragma omp parallel for schedule(static)
+  for (int b = 0; b < B; ++b)
+    fbifft2dSmallPlane(cplx + b * inPlane, N, h, w, padL, padU, real + b * outPlane, true);
+  return 0;
+}
+
+// The per-frequency contraction on packed spectra [..][..][N/2][N]: rows 1..N/2-1
+// as orc_transpose_mm; row 0 by the product rule of the fused kernels
+// (FFTIteratedConvolution.cuh:161-186 for a * conj(b), :317-337 for a * b, :483-504
+// for the unpacking): with other = P[N - x], F0 = 0.5 (conj(other) + P),
+// FH = 0.5 transpose(conj(conj(other) - P)), the rows multiply separately and
+// acc += out0 + transpose(conj(outH)); lane 0 multiplies its two real pairs
+// component by component.  op() conjugates the unpacked values.
+void orc_transpose_mm_packed(const float* A, const float* B, float* C, int I, int J, int K, int N,
+                             int conjA, int conjB, int accumulate, float invNorm) {
+  const cf* a = reinterpret_cast<const cf*>(A);
+  const cf* b = reinterpret_cast<const cf*>(B);
+  cf* c = reinterpret_cast<cf*>(C);
+  const int XY = N / 2 * N;
+#pragma omp parallel for collapse(2) schedule(static)
+  for (int i = 0; i < I; ++i) {
+    for (int j = 0; j < J; ++j) {
+      for (int xy = 0; xy < XY; ++xy) {
+        cf acc = accumulate ? c[((size_t)i * J + j) * XY + xy] : mk(0.0f);
+        for (int k = 0; k < K; ++k) {
+          const cf* ap = conjA ? a + ((size_t)k * I + i) * XY : a + ((size_t)i * K + k) * XY;
+          const cf* bp = conjB ? b + ((size_t)j * K + k) * XY : b + ((size_t)k * J + j) * XY;
+          cf av = ap[xy], bv = bp[xy];
+          if (xy >= N) {
+            if (conjA) av = conj(av);
+            if (conjB) bv = conj(bv);
+            acc = av * bv + acc;
+          } else if (xy > 0) {
+            cf oa = ap[N - xy], ob = bp[N - xy];
+            cf a0 = mk(0.5f) * (conj(oa) + av);
+            cf aH = mk(0.5f) * swp(conj(conj(oa) - av));
+            cf b0 = mk(0.5f) * (conj(ob) + bv);
+            cf bH = mk(0.5f) * swp(conj(conj(ob) - bv));
+            if (conjA) { a0 = conj(a0); aH = conj(aH); }
+            if (conjB) { b0 = conj(b0); bH = conj(bH); }
+            cf out0 = a0 * b0;
+            cf outH = aH * bH;
+            acc = acc + (out0 + swp(conj(outH)));
+          } else {
+            acc = acc + mk(av.re * bv.re, av.im * bv.im);
+          }
+        }
+        acc.re *= invNorm;
+        acc.im *= invNorm;
+        c[((size_t)i * J + j) * XY + xy] = acc;
+      }
+    }
+  }
 }
 
 // transposeMM (MM-inl.cuh:188-196 semantics, :302-326 accumulation order and

@@ -186,9 +186,14 @@ int main() {
   HIP_OK(hipMalloc((void**)&dback, x.size() * 4));
   HIP_OK(hipMemcpy(dx, x.data(), x.size() * 4, hipMemcpyHostToDevice));
 
-  int rs[3] = {B, N, N}, cs[4] = {B, nc, N, 2};
-  DeviceTensor<float, 3> real(dx, rs), back(dback, rs);
-  DeviceTensor<float, 4> spec(dspec, cs);
+  // operands arrive as [batch][planes][h][w]; the callers flatten batch x planes with
+  // downcastOuter before the 2D transforms
+  int rs4[4] = {1, B, N, N}, cs5[5] = {1, B, nc, N, 2}, rs[3] = {B, N, N};
+  DeviceTensor<float, 4> real4(dx, rs4);
+  DeviceTensor<float, 5> spec5(dspec, cs5);
+  DeviceTensor<float, 3> real = real4.downcastOuter<3>(), back(dback, rs);
+  DeviceTensor<float, 4> spec = spec5.downcastOuter<4>();
+  if (real.getSize(0) != B || spec.getSize(1) != nc || !real.isContiguous()) return 3;
   if (fbfft::fbfft2D<1>(real, spec) != FBFFTParameters::Success) return 3;
   int ccs[3] = {B, nc, N};
   DeviceTensor<Complex, 3> cspec(reinterpret_cast<Complex*>(dspec), ccs);

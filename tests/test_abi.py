@@ -94,6 +94,17 @@ def test_cpp_facade_compiles_against_reference_include_paths():
     assert os.path.exists(os.path.join(ROOT, "tests", "cpp", "facade_check"))
 
 
+def test_cpp_device_tensor_and_complex_host_arithmetic():
+    """tests/cpp/tensor_check.cpp: sizes / strides of downcast, upcast, transpose, permute,
+    view and cast, and Complex's operators, against hand-written expectations (host only)."""
+    import subprocess
+    subprocess.check_call(["make", "-C", os.path.join(ROOT, "tests", "cpp"), "-B", "tensor_check"],
+                          stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL)
+    out = subprocess.run([os.path.join(ROOT, "tests", "cpp", "tensor_check")], capture_output=True,
+                         text=True)
+    assert out.returncode == 0 and out.stdout.strip() == "OK", out.stdout
+
+
 def _fake_tensor(shape, base=0x10000000):
     """fbfft_tensor over memory that is never touched: the tile builder only does
     address arithmetic."""

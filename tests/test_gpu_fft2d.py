@@ -97,7 +97,10 @@ def test_error_codes():
     assert F.fbfft2D(real, torch.zeros((4, 17, 32, 2), device=d)) == F.Success
     assert F.fbfft2D(real, torch.zeros((4, 129, 256, 2), device=d)) == F.UnsupportedSize
     assert F.fbfft2D(real, torch.zeros((4, 7, 12, 2), device=d)) == F.UnsupportedSize
-    assert F.fbfft2D(real, torch.zeros((4, 16, 32, 2), device=d)) == F.UnsupportedSize
+    assert F.fbfft2D(real, torch.zeros((4, 15, 32, 2), device=d)) == F.UnsupportedSize
+    assert F.fbfft2D(real, torch.zeros((4, 16, 32, 2), device=d)) == F.Success  # packed rows
+    assert F.fbfft2D(torch.zeros((4, 64, 64), device=d),
+                     torch.zeros((4, 32, 64, 2), device=d)) == F.UnsupportedSize  # N <= 32 only
     assert F.fbfft2D(real, torch.zeros((3, 17, 32, 2), device=d)) == F.UnsupportedDimension
     assert F.fbfft2D(real, torch.zeros((4, 17, 32), device=d)) == F.UnsupportedDimension
     assert F.fbfft2D(torch.zeros((4, 40, 32), device=d),

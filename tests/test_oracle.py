@@ -303,3 +303,83 @@ def test_brute_force_tiny(oracle):
     want = np.array([[sum(x[b, n] * np.exp(-2j * np.pi * k * n / 8) for n in range(8))
                       for k in range(5)] for b in range(3)])
     assert rel(c(out), want) < TOL
+
+
+# ---- packed spectrum format (FFT2D32.cuh:421-427, :302-316; product rule of
+# FFTIteratedConvolution.cuh:161-186) ----
+
+from packed_util import as_float, pack, unpack  # noqa: E402
+
+
+def test_pack_unpack_helpers_are_inverse():
+    rng = np.random.default_rng(3)
+    X = rng.standard_normal((2, 16, 16))
+    U = np.fft.fft2(X)[:, :9, :]
+    assert np.allclose(unpack(pack(U)), U, atol=1e-12)
+    P = rng.standard_normal((3, 8, 16)) + 1j * rng.standard_normal((3, 8, 16))
+    assert np.allclose(pack(unpack(P)), P, atol=1e-12)
+
+
+@pytest.mark.parametrize("N,h,w,padL,padU", [(8, 8, 8, 0, 0), (16, 16, 16, 0, 0), (32, 32, 32, 0, 0),
+                                              (32, 27, 27, 0, 0), (16, 5, 7, 3, 2), (8, 3, 3, 5, 4)])
+def test_packed_forward_is_the_packed_dft(oracle, N, h, w, padL, padU):
+    rng = np.random.default_rng(N + h)
+    x = rng.standard_normal((5, h, w)).astype(np.float32)
+    rc, got = oracle.fbfft2d_packed(x, N, padL, padU)
+    assert rc == 0 and got.shape == (5, N // 2, N, 2)
+    want = pack(spec2d(embed(x.astype(np.float64), N, padL, padU), N))
+    assert rel(c(got), want) < TOL
+    # and against the transcription of the unpacked store
+    _, unp = oracle.fbfft2d(x, N, padL, padU)
+    assert rel(unpack(c(got)), c(unp)) < TOL
+
+
+@pytest.mark.parametrize("N,h,w,padL,padU", [(8, 8, 8, 0, 0), (16, 16, 16, 0, 0), (32, 32, 32, 0, 0),
+                                              (32, 23, 23, 0, 0), (16, 9, 6, 2, 5)])
+def test_packed_inverse_inverts_the_packed_dft(oracle, N, h, w, padL, padU):
+    rng = np.random.default_rng(7 * N + w)
+    X = rng.standard_normal((4, N, N))
+    P = as_float(pack(spec2d(X, N)))
+    rc, back = oracle.fbifft2d_packed(P, h, w, padL, padU)
+    assert rc == 0
+    assert rel(back, N * N * X[:, padU:padU + h, padL:padL + w]) < TOL
+
+
+@pytest.mark.parametrize("conjA,conjB", [(False, True), (True, False), (False, False)])
+@pytest.mark.parametrize("N", [8, 16, 32])
+def test_packed_contraction_is_the_contraction_of_the_unpacked_spectra(oracle, N, conjA, conjB):
+    rng = np.random.default_rng(100 + N)
+    I, J, K = 3, 4, 5
+
+    def spectra(d0, d1):
+        return as_float(pack(spec2d(rng.standard_normal((d0 * d1, N, N)), N)).reshape(d0, d1, N // 2, N))
+
+    A = spectra(*((K, I) if conjA else (I, K)))
+    B = spectra(*((J, K) if conjB else (K, J)))
+    got = oracle.transpose_mm_packed(A, B, conjA, conjB, 0.25)
+    UA, UB = unpack(c(A)), unpack(c(B))
+    a = np.conj(UA).transpose(1, 0, 2, 3) if conjA else UA
+    b = np.conj(UB).transpose(1, 0, 2, 3) if conjB else UB
+    want = 0.25 * np.einsum("ikyx,kjyx->ijyx", a, b)
+    assert rel(unpack(c(got)), want) < TOL
+    assert rel(c(got), pack(want)) < TOL
+    # Accumulate: invNorm scales the accumulated-into value as well (MM-inl.cuh:322-324)
+    C0 = spectra(I, J)
+    acc = oracle.transpose_mm_packed(A, B, conjA, conjB, 0.25, C=C0)
+    assert rel(c(acc), pack(want + 0.25 * unpack(c(C0)))) < TOL
+
+
+def test_packed_layer_equals_direct_correlation(oracle):
+    """packed FFT -> packed contraction -> packed inverse = fp64 valid correlation."""
+    N, Nb, Cin, Cout, H, k = 16, 2, 3, 4, 13, 4
+    rng = np.random.default_rng(9)
+    x = rng.standard_normal((Nb, Cin, H, H)).astype(np.float32)
+    w = rng.standard_normal((Cout, Cin, k, k)).astype(np.float32)
+    _, X = oracle.fbfft2d_packed(x.reshape(-1, H, H), N)
+    _, W = oracle.fbfft2d_packed(w.reshape(-1, k, k), N)
+    X = X.reshape(Nb, Cin, N // 2, N, 2)
+    W = W.reshape(Cout, Cin, N // 2, N, 2)
+    O = oracle.transpose_mm_packed(X, W, False, True, 1.0 / (N * N))
+    o = H - k + 1
+    _, out = oracle.fbifft2d_packed(O.reshape(-1, N // 2, N, 2), o, o)
+    assert rel(out.reshape(Nb, Cout, o, o), oracle.corr2d_valid(x, w)) < 1e-4
