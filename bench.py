@@ -306,6 +306,38 @@ def run_only(name, steps, warmup, F, synth, torch, dev):
         return {"only": name, "us": round(t * 1e6, 2),
                 "GBps": round(b * (4 * n + 8 * (n // 2 + 1)) / t / 1e9, 1)}
     extra = {}
+    if name == "iter4":
+        # configs[4] updateOutput through the fused tiled kernel only
+        x4 = synth.uniform((16, 32, 256, 256), seed=40, device=dev)
+        w4 = synth.normal((32, 32, 9, 9), seed=41, std=0.05, device=dev)
+        o4 = torch.empty((16, 32, 248, 248), device=dev)
+        ins, outs, n = F.make_tile_grid(x4, o4, 9, 9, 32)
+        vw4 = F.view(w4)
+        stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+        def tiled():
+            rc = F.lib().fbfft_iterated_conv(32, ctypes.c_void_p(ins.data_ptr()),
+                                             ctypes.c_void_p(outs.data_ptr()), ctypes.byref(vw4), 0,
+                                             ctypes.c_float(1.0), 16, n, stream)
+            assert rc == 1
+        _, t = timed(tiled, steps, warmup, torch)
+        return {"only": name, "us": round(t * 1e6, 2)}
+    if name == "conv4":
+        # configs[4] updateOutput through the layer entry point (overlap-tiled pipeline)
+        x4 = synth.uniform((16, 32, 256, 256), seed=40, device=dev)
+        w4 = synth.normal((32, 32, 9, 9), seed=41, std=0.05, device=dev)
+        o4 = torch.empty((16, 32, 248, 248), device=dev)
+        ws4 = torch.empty(F.conv_workspace_image(0, 16, 32, 32, 256, 256, 9, 9, 32),
+                          dtype=torch.uint8, device=dev)
+        stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+        v4 = (F.view(x4), F.view(w4), F.view(o4))
+
+        def layer():
+            rc = F.lib().fbfft_conv_fprop(ctypes.byref(v4[0]), ctypes.byref(v4[1]), ctypes.byref(v4[2]),
+                                          32, ctypes.c_void_p(ws4.data_ptr()), ws4.numel(), stream)
+            assert rc == 0
+        _, t = timed(layer, steps, warmup, torch)
+        return {"only": name, "us": round(t * 1e6, 2)}
     if name == "mm":
         A = synth.normal((128, 64, 17, 32, 2), seed=30, device=dev)
         Bm = synth.normal((192, 64, 17, 32, 2), seed=31, device=dev)
@@ -344,7 +376,7 @@ def main():
     ap.add_argument("--no-extra", action="store_true", help="skip the informative extra configs")
     ap.add_argument("--only", default=None,
                     choices=["r2c32", "c2r32", "r2c64", "c2r64", "r2c128", "c2r128", "mm", "conv",
-                             "iterconv", "r2c1d", "c2r1d"],
+                             "iterconv", "iter4", "conv4", "r2c1d", "c2r1d"],
                     help="run just this workload --steps times (for rocprofv3) and print its timing")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="only run a plain 256 MiB device-to-device copy 20 times: the known-size "

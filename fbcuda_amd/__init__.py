@@ -48,7 +48,7 @@ EXPORTS = (
     "fbfft_r2c_1d", "fbfft_c2r_1d", "fbfft_r2c_2d", "fbfft_c2c_2d_pass2", "fbfft_c2r_2d",
     "fbfft_c2c_2d_inverse_pass1", "fbfft_transpose_mm", "fbfft_transpose_mm_packed", "fbfft_iterated_conv", "fbfft_make_tiles",
     "fbfft_make_tiles_for_pass",
-    "fbfft_conv_workspace", "fbfft_conv_fprop_workspace", "fbfft_conv_fprop", "fbfft_conv_bprop",
+    "fbfft_conv_workspace", "fbfft_conv_workspace_image", "fbfft_conv_fprop_workspace", "fbfft_conv_fprop", "fbfft_conv_bprop",
     "fbfft_conv_accgrad", "fbfft_conv_fprop_static", "fbfft_error_string",
     "fbfft_twiddle_table",
 )
@@ -87,6 +87,8 @@ def lib():
         L.fbfft_conv_fprop.argtypes = [tp, tp, tp, ctypes.c_int, vp, ctypes.c_size_t, vp]
         L.fbfft_conv_workspace.argtypes = [ctypes.c_int] * 5
         L.fbfft_conv_workspace.restype = ctypes.c_size_t
+        L.fbfft_conv_workspace_image.argtypes = [ctypes.c_int] * 9
+        L.fbfft_conv_workspace_image.restype = ctypes.c_size_t
         L.fbfft_conv_bprop.argtypes = [tp, tp, tp, ctypes.c_int, vp, ctypes.c_size_t, vp]
         L.fbfft_conv_accgrad.argtypes = [tp, tp, tp, ctypes.c_int, ctypes.c_float, ctypes.c_int, vp,
                                          ctypes.c_size_t, vp]
@@ -269,6 +271,12 @@ def conv_fprop_static(input, weight, output, fftSize, stream=None):
 def conv_workspace(pass_, batch, cin, cout, fftSize):
     """Workspace bytes of pass 0 (conv_fprop), 1 (conv_bprop) or 2 (conv_accgrad)."""
     return lib().fbfft_conv_workspace(int(pass_), batch, cin, cout, fftSize)
+
+
+def conv_workspace_image(pass_, batch, cin, cout, H, W, kH, kW, fftSize):
+    """Workspace bytes of a pass for input extents H x W (images larger than the transform
+    are overlap-tiled when fftSize <= 32)."""
+    return lib().fbfft_conv_workspace_image(int(pass_), batch, cin, cout, H, W, kH, kW, fftSize)
 
 
 def conv_bprop(gradOutput, weight, gradInput, fftSize, workspace, stream=None):

@@ -245,7 +245,9 @@ int checkConvShapes(const fbfft_tensor* input, const fbfft_tensor* weight,
   const int Cout = weight->size[0], kH = weight->size[2], kW = weight->size[3];
   if (weight->size[1] != Cin || output->size[0] != B || output->size[1] != Cout)
     return FBFFT_UNSUPPORTED_DIMENSION;
-  if (H > N || W > N || kH > H || kW > W) return FBFFT_UNSUPPORTED_SIZE;
+  if (kH > H || kW > W || kH > N || kW > N) return FBFFT_UNSUPPORTED_SIZE;
+  // images larger than the transform are overlap-tiled by the 8 / 16 / 32-point path only
+  if ((H > N || W > N) && N > 32) return FBFFT_UNSUPPORTED_SIZE;
   if (output->size[2] != H - kH + 1 || output->size[3] != W - kW + 1)
     return FBFFT_UNSUPPORTED_DIMENSION;
   return FBFFT_SUCCESS;
@@ -257,8 +259,10 @@ int convPass(int pass, const fbfft_tensor* input, const fbfft_tensor* weight,
   const int rc = checkConvShapes(input, weight, output, N);
   if (rc != FBFFT_SUCCESS) return rc;
   if (empty(input) || empty(weight) || empty(output)) return FBFFT_SUCCESS;
-  if (!workspace || !aligned(workspace, 256) ||
-      workspaceBytes < fbfft_conv_workspace(pass, input->size[0], input->size[1], weight->size[0], N))
+  const size_t need = fbfft_conv_workspace_image(pass, input->size[0], input->size[1],
+                                                 weight->size[0], input->size[2], input->size[3],
+                                                 weight->size[2], weight->size[3], N);
+  if (!workspace || !aligned(workspace, 256) || need == 0 || workspaceBytes < need)
     return FBFFT_UNSUPPORTED_DIMENSION;
   const fbfft_tensor *x, *y, *out;
   if (pass == 0) {
@@ -274,10 +278,17 @@ int convPass(int pass, const fbfft_tensor* input, const fbfft_tensor* weight,
 
 }  // namespace
 
-extern "C" size_t fbfft_conv_workspace(int pass, int batch, int cin, int cout, int fftSize) {
+extern "C" size_t fbfft_conv_workspace_image(int pass, int batch, int cin, int cout, int H, int W,
+                                             int kH, int kW, int fftSize) {
   if (pass < 0 || pass > 2 || batch <= 0 || cin <= 0 || cout <= 0) return 0;
   if (!convSizeOk(fftSize)) return 0;
-  return convWorkspaceBytes(pass, fftSize, batch, cin, cout);
+  if (kH < 1 || kW < 1 || kH > H || kW > W || kH > fftSize || kW > fftSize) return 0;
+  if ((H > fftSize || W > fftSize) && fftSize > 32) return 0;
+  return convWorkspaceBytes(pass, fftSize, batch, cin, cout, H, W, kH, kW);
+}
+
+extern "C" size_t fbfft_conv_workspace(int pass, int batch, int cin, int cout, int fftSize) {
+  return fbfft_conv_workspace_image(pass, batch, cin, cout, fftSize, fftSize, 1, 1, fftSize);
 }
 
 extern "C" size_t fbfft_conv_fprop_workspace(int batch, int cin, int cout, int fftSize) {

@@ -73,7 +73,8 @@ int launchTwoPass(int N, int mode, float* src, long s0, long s1, long s2, float*
                   long d1, long d2, int B, int h, int w, int padL, int padU, hipStream_t s);
 
 // pass 0 / 1 / 2 = forward, input gradient, weight gradient (x, y, out as in conv_pipeline.hip)
-size_t convWorkspaceBytes(int pass, int N, int B, int Cin, int Cout);
+// H, W: the layer's input extents (larger than N: overlap tiling, N <= 32 only)
+size_t convWorkspaceBytes(int pass, int N, int B, int Cin, int Cout, int H, int W, int kH, int kW);
 int launchConvPass(int pass, int N, float* x, const int* xStride, const int* xSize, float* y,
                    const int* yStride, const int* ySize, float* out, const int* outStride,
                    const int* outSize, float scale, bool accumulate, void* workspace,

@@ -55,12 +55,47 @@ struct BMCfg {
   static constexpr int BINS = (H + 1) * N;
 };
 
+// A family of planes indexed by (row, k).  Plain: plane (row, k) is the h x w window at
+// base + row*sRow + k*sK.  Tiled (images larger than the transform): one of the two
+// indices is the composite (image, tileY, tileX), image-major; its stride is the
+// image stride, h x w is the whole image, and tile (ty, tx) is the winH x winW
+// window at (orgY + ty*stepY, orgX + tx*stepX) clipped to the image - rows and
+// columns clipped off above / left become the plane's padU / padL, so the window
+// keeps its place inside the FFT plane.  padU0 / padL0 shift every window further
+// (where a cropped result sits inside the inverse transform's plane).
 struct PlaneSet {
-  float* base;      // plane (row, k) starts at base + row*sRow + k*sK
+  float* base;
   long sRow, sK;
   int sy, sx, h, w;
   int R, K;         // valid rows / k
+  int tiled;        // 0: plain, 1: row is the composite index, 2: k is
+  int tilesY, tilesX, stepY, stepX, orgY, orgX, winH, winW;
+  int padU0, padL0;
 };
+
+struct PlaneWindow {
+  float* p;
+  int h, w, padL, padU;
+};
+
+__device__ __forceinline__ PlaneWindow planeWindow(const PlaneSet& ps, int row, int k) {
+  if (ps.tiled == 0)
+    return PlaneWindow{ps.base + (long)row * ps.sRow + (long)k * ps.sK, ps.h, ps.w, ps.padL0,
+                       ps.padU0};
+  const int comp = ps.tiled == 1 ? row : k, other = ps.tiled == 1 ? k : row;
+  const long sImg = ps.tiled == 1 ? ps.sRow : ps.sK, sOther = ps.tiled == 1 ? ps.sK : ps.sRow;
+  const int perImage = ps.tilesY * ps.tilesX;
+  const int img = comp / perImage, t = comp % perImage;
+  const int y0 = ps.orgY + (t / ps.tilesX) * ps.stepY, x0 = ps.orgX + (t % ps.tilesX) * ps.stepX;
+  const int ya = max(y0, 0), xa = max(x0, 0);
+  PlaneWindow win;
+  win.p = ps.base + (long)img * sImg + (long)other * sOther + (long)ya * ps.sy + (long)xa * ps.sx;
+  win.h = min(y0 + ps.winH, ps.h) - ya;
+  win.w = min(x0 + ps.winW, ps.w) - xa;
+  win.padU = ps.padU0 + ya - y0;
+  win.padL = ps.padL0 + xa - x0;
+  return win;
+}
 
 // ---- 1. planes -> S[bin][k][row] ----
 // PAIRS: every plane of the set passes windowMovesAsPairs() (8-byte words per row)
@@ -78,8 +113,8 @@ __global__ __launch_bounds__(kT) void forwardBinMajor(PlaneSet ps, float2* S, in
 
   c32 z0[H], z1[H];
   if (row < ps.R && k < ps.K) {
-    loadColumnsWindow<N, PAIRS>(ps.base + (long)row * ps.sRow + (long)k * ps.sK, ps.sy, ps.sx,
-                                ps.h, ps.w, 0, 0, l, z0, z1);
+    const PlaneWindow win = planeWindow(ps, row, k);
+    loadColumnsWindow<N, PAIRS>(win.p, ps.sy, ps.sx, win.h, win.w, win.padL, win.padU, l, z0, z1);
   } else {
 #pragma unroll
     for (int j = 0; j < H; ++j) z0[j] = z1[j] = c32{0.f, 0.f};
@@ -167,9 +202,11 @@ __global__ __launch_bounds__(kT) void inverseBinMajor(const float2* Cs, int I, i
   c32 z0[H], z1[H];
   columnPassInverse<N>(plane, l, z0, z1);
   const int j = j0 + s;
-  if (j < out.K)  // out.K: number of valid output planes along j
-    storeColumnsWindow<N, ACC>(out.base + (long)i * out.sRow + (long)j * out.sK, out.sy, out.sx,
-                               out.h, out.w, 0, 0, l, z0, z1, scale);
+  if (j < out.K) {  // out.K: number of valid output planes along j
+    const PlaneWindow win = planeWindow(out, i, j);
+    storeColumnsWindow<N, ACC>(win.p, out.sy, out.sx, win.h, win.w, win.padL, win.padU, l, z0, z1,
+                               scale);
+  }
 }
 
 // ---- 2. batched complex GEMM, bin-major ----
@@ -358,6 +395,7 @@ int runPipeline(PlaneSet x, PlaneSet y, PlaneSet out, bool conjY, float scale, b
     xSign = conjY ? -1.0f : 1.0f;
     ySign = -1.0f;
     std::swap(out.sRow, out.sK);
+    if (out.tiled) out.tiled = 3 - out.tiled;
   }
   const int I = x.R, J = y.R, K = x.K;
   out.R = I;
@@ -368,8 +406,10 @@ int runPipeline(PlaneSet x, PlaneSet y, PlaneSet out, bool conjY, float scale, b
   float2* SC = SB + (size_t)bins * Kp * Jp;
 
   auto forward = [&](const PlaneSet& p, float2* S, int Rp, float sign) {
-    const bool pairs = windowMovesAsPairs(p.base, p.sy, p.sx, p.w, 0) && p.sRow % 2 == 0 &&
-                       p.sK % 2 == 0;
+    // every window of the set starts on an 8-byte boundary with an even width and pad
+    const bool pairs = windowMovesAsPairs(p.base, p.sy, p.sx, p.w, p.padL0) && p.sRow % 2 == 0 &&
+                       p.sK % 2 == 0 &&
+                       (!p.tiled || ((p.stepX | p.orgX | p.winW) & 1) == 0);
     if (pairs)
       forwardBinMajor<N, 1><<<dim3(Rp / SL, Kp), dim3(kT), 0, s>>>(p, S, Rp, Kp, sign);
     else
@@ -407,8 +447,33 @@ int runPipeline(PlaneSet x, PlaneSet y, PlaneSet out, bool conjY, float scale, b
 }
 
 PlaneSet planes(float* base, const int* stride, const int* size, int rowDim, int kDim) {
-  return PlaneSet{base, stride[rowDim], stride[kDim], stride[2], stride[3], size[2], size[3],
-                  size[rowDim], size[kDim]};
+  PlaneSet p{};
+  p.base = base;
+  p.sRow = stride[rowDim];
+  p.sK = stride[kDim];
+  p.sy = stride[2];
+  p.sx = stride[3];
+  p.h = size[2];
+  p.w = size[3];
+  p.R = size[rowDim];
+  p.K = size[kDim];
+  return p;
+}
+
+// Cuts the images of p into tilesY x tilesX windows; the index of dimension 0 (the
+// image) - p's row or k - becomes the composite (image, tileY, tileX).
+void tile(PlaneSet& p, bool imageIsRow, int tilesY, int tilesX, int stepY, int stepX, int orgY,
+          int orgX, int winH, int winW) {
+  p.tiled = imageIsRow ? 1 : 2;
+  p.tilesY = tilesY;
+  p.tilesX = tilesX;
+  p.stepY = stepY;
+  p.stepX = stepX;
+  p.orgY = orgY;
+  p.orgX = orgX;
+  p.winH = winH;
+  p.winW = winW;
+  (imageIsRow ? p.R : p.K) *= tilesY * tilesX;
 }
 
 template <int N>
@@ -419,17 +484,33 @@ int runPass(int pass, const PlaneSet& x, const PlaneSet& y, const PlaneSet& out,
 
 }  // namespace
 
-// (I, J, K) of a pass for batch B and Cin / Cout planes
+// Tiles per image of a pass: 1 when the image fits the transform.  The forward pass
+// and the weight gradient walk the OUTPUT in disjoint (N-kH+1) x (N-kW+1) windows,
+// the input gradient walks the INPUT (the tensor it writes) in such windows.
+static void tileGrid(int pass, int N, int H, int W, int kH, int kW, int* tilesY, int* tilesX) {
+  *tilesY = *tilesX = 1;
+  if (H <= N && W <= N) return;
+  const int stepY = N - kH + 1, stepX = N - kW + 1;
+  const int spanY = pass == 1 ? H : H - kH + 1, spanX = pass == 1 ? W : W - kW + 1;
+  *tilesY = ceilDiv(spanY, stepY);
+  *tilesX = ceilDiv(spanX, stepX);
+}
+
+// (I, J, K) of a pass for batch B (times the tiles per image) and Cin / Cout planes
 static void passDims(int pass, int B, int Cin, int Cout, int* I, int* J, int* K) {
   if (pass == 0) { *I = B; *J = Cout; *K = Cin; }
   else if (pass == 1) { *I = B; *J = Cin; *K = Cout; }
   else { *I = Cin; *J = Cout; *K = B; }
 }
 
-size_t convWorkspaceBytes(int pass, int N, int B, int Cin, int Cout) {
+size_t convWorkspaceBytes(int pass, int N, int B, int Cin, int Cout, int H, int W, int kH,
+                          int kW) {
   if (N > 32) return convSplitWorkspaceBytes(pass, N, B, Cin, Cout);
+  int ty, tx;
+  tileGrid(pass, N, H, W, kH, kW, &ty, &tx);
+  if ((long)B * ty * tx > (1L << 30)) return 0;
   int I, J, K;
-  passDims(pass, B, Cin, Cout, &I, &J, &K);
+  passDims(pass, B * ty * tx, Cin, Cout, &I, &J, &K);
   size_t n = N == 8 ? workspaceFloat2<8>(I, J, K)
                     : N == 16 ? workspaceFloat2<16>(I, J, K) : workspaceFloat2<32>(I, J, K);
   return n * sizeof(float2);
@@ -438,7 +519,9 @@ size_t convWorkspaceBytes(int pass, int N, int B, int Cin, int Cout) {
 // pass 0: x = input [B][Cin][H][W], y = weight [Cout][Cin][kH][kW], out = output [B][Cout][oH][oW]
 // pass 1: x = gradOutput [B][Cout][oH][oW], y = weight, out = gradInput [B][Cin][H][W]
 // pass 2: x = input, y = gradOutput, out = gradWeight [Cout][Cin][kH][kW]
-// strides in floats
+// strides in floats.  Images larger than the transform (N <= 32 only) are cut into
+// overlapping windows that ride through the same three kernels as extra rows
+// (passes 0 and 1) or extra reduction steps (pass 2).
 int launchConvPass(int pass, int N, float* x, const int* xStride, const int* xSize, float* y,
                    const int* yStride, const int* ySize, float* out, const int* outStride,
                    const int* outSize, float scale, bool accumulate, void* workspace,
@@ -459,6 +542,29 @@ int launchConvPass(int pass, int N, float* x, const int* xStride, const int* xSi
     px = planes(x, xStride, xSize, 1, 0);
     py = planes(y, yStride, ySize, 1, 0);
     po = planes(out, outStride, outSize, 1, 0);
+  }
+  const int* in = pass == 1 ? outSize : xSize;    // the layer's input / gradInput extents
+  const int* wt = pass == 2 ? outSize : ySize;    // the filter extents
+  const int H = in[2], W = in[3], kH = wt[2], kW = wt[3];
+  int ty, tx;
+  tileGrid(pass, N, H, W, kH, kW, &ty, &tx);
+  if (ty * tx > 1) {
+    const int stepY = N - kH + 1, stepX = N - kW + 1;
+    if (pass == 0) {
+      tile(px, true, ty, tx, stepY, stepX, 0, 0, N, N);
+      tile(po, true, ty, tx, stepY, stepX, 0, 0, stepY, stepX);
+    } else if (pass == 1) {
+      // gradInput rows y0 .. y0+step-1 are a full convolution over gradOutput rows
+      // y0-(kH-1) .. y0+step-1; the result for row y0 then sits in plane row kH-1,
+      // clear of the circular wrap-around
+      tile(px, true, ty, tx, stepY, stepX, -(kH - 1), -(kW - 1), N, N);
+      tile(po, true, ty, tx, stepY, stepX, 0, 0, stepY, stepX);
+      po.padU0 = kH - 1;
+      po.padL0 = kW - 1;
+    } else {
+      tile(px, false, ty, tx, stepY, stepX, 0, 0, N, N);
+      tile(py, false, ty, tx, stepY, stepX, 0, 0, stepY, stepX);
+    }
   }
   float2* ws = static_cast<float2*>(workspace);
   switch (N) {

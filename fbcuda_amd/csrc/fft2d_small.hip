@@ -327,6 +327,10 @@ int computeUnits() {
   return n;
 }
 
+// (Measured across the switch, 32 x 32 R2C, us per launch paired / unpaired: 9216 planes
+// 16.6 / 16.0, 10240 17.0 / 17.4, 12288 17.8 / 19.5, 14336 19.1 / 22.0, 16384 22.7 / 24.1;
+// a variant that keeps one full round of waves and gives only some of them a second
+// group was no better: 16.7, 17.0, 18.9, 20.3, 22.8.)
 template <int N>
 bool pairGroups(int groups) {
   constexpr int ldsBytes = SmallCfg<N>::P * SmallCfg<N>::PS * (int)sizeof(c32);

@@ -189,17 +189,29 @@ size_t fbfft_make_tiles_for_pass(int pass, const fbfft_tensor* input, const fbff
  * sequences that the reference's external callers compose from the primitives
  * above, one entry point per pass of the role table at MM-inl.cuh:188-196.
  * Shapes throughout: input / gradInput [B][Cin][H][W], weight / gradWeight
- * [Cout][Cin][kH][kW], output / gradOutput [B][Cout][H-kH+1][W-kW+1], with
- * H, W <= fftSize in {8,16,32,64,128}.  Valid cross-correlation, no kernel flip.
+ * [Cout][Cin][kH][kW], output / gradOutput [B][Cout][H-kH+1][W-kW+1], fftSize in
+ * {8,16,32,64,128}, kH, kW <= fftSize.  Valid cross-correlation, no kernel flip.
  * Sizes up to 32 hand bin-major spectra between three fused kernels; 64 and 128
- * run fbfft2D -> transposeMM -> fbifft2D on plane-major spectra in the workspace.
- * workspace: device memory of at least fbfft_conv_workspace() bytes for that
- * pass, 256-byte aligned; its contents need not survive between calls. */
+ * run fbfft2D -> transposeMM -> fbifft2D on plane-major spectra in the workspace
+ * and need H, W <= fftSize.  With fftSize <= 32 the image may be larger than the
+ * transform: it is then cut into overlapping fftSize x fftSize windows whose
+ * origins advance by fftSize-kH+1 rows / fftSize-kW+1 columns (the tiling of
+ * FFTIteratedConvolution, fbfft/FFTIteratedConvolution.cuh:71-88), and the
+ * windows ride through the same three kernels as extra images (forward pass,
+ * input gradient) or extra reduction steps (weight gradient).
+ * workspace: device memory of at least fbfft_conv_workspace_image() bytes for
+ * that pass and image size (fbfft_conv_workspace() when H, W <= fftSize),
+ * 256-byte aligned; its contents need not survive between calls. */
 
 /* Bytes of workspace for pass 0 (fprop), 1 (bprop) or 2 (accgrad): the values of
  * FFTConvolutionPassFFI (fbfft/FFTIteratedConvolution.cuh:616-622).  0 when the
  * arguments are not supported. */
 size_t fbfft_conv_workspace(int pass, int batch, int cin, int cout, int fftSize);
+
+/* The same for a layer with input extents H x W and a kH x kW filter; equal to
+ * fbfft_conv_workspace when H, W <= fftSize. */
+size_t fbfft_conv_workspace_image(int pass, int batch, int cin, int cout, int H, int W, int kH,
+                                  int kW, int fftSize);
 
 /* Same as fbfft_conv_workspace(0, ...). */
 size_t fbfft_conv_fprop_workspace(int batch, int cin, int cout, int fftSize);
