@@ -269,6 +269,29 @@ def conv_extras(F, synth, torch, dev, extra):
     _, t = timed(tiled, 30, 20, torch)
     extra["iterated_conv_configs4_ms_per_iter"] = round(t * 1e3, 4)
     extra["iterated_conv_configs4_direct_equiv_TFLOPs"] = round(163.3e9 / t / 1e12, 1)
+    # the same layer through the convolution-layer entry point: the 121 windows per image
+    # ride through the bin-major pipeline (spectra in a workspace) instead of the fused kernel
+    ws4 = torch.empty(F.conv_workspace_image(0, 16, 32, 32, 256, 256, 9, 9, 32), dtype=torch.uint8,
+                      device=dev)
+    v4 = (F.view(x4), F.view(w4), F.view(o4))
+
+    def layer4():
+        if L.fbfft_conv_fprop(ctypes.byref(v4[0]), ctypes.byref(v4[1]), ctypes.byref(v4[2]), 32,
+                              ctypes.c_void_p(ws4.data_ptr()), ws4.numel(), stream) != 0:
+            raise RuntimeError("fbfft_conv_fprop (tiled) failed")
+    _, t = timed(layer4, 60, 40, torch)
+    mid, low = spread(layer4, 60, torch)
+    extra["conv_layer_configs4_ms_per_iter"] = round(t * 1e3, 4)
+    extra["conv_layer_configs4_ms_per_iter_median"] = round(mid * 1e3, 4)
+    extra["conv_layer_configs4_ms_per_iter_min"] = round(low * 1e3, 4)
+    extra["conv_layer_configs4_direct_equiv_TFLOPs"] = round(163.3e9 / t / 1e12, 1)
+    # 260.5 MB of algorithmic traffic (input + filters + output) against the HBM peak
+    extra["conv_layer_configs4_roofline"] = {
+        "bound": "hbm", "achieved": round(260.5e6 / t / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+        "frac": round(260.5e6 / t / 1e9 / HBM_PEAK_GBS, 4), "algorithmic_bytes": 260500000,
+        "traffic": profile_figure("conv_pipeline_configs4.md", "traffic_bytes_per_iteration"),
+        "workload": "configs[4]: 16x32x256x256 * 32x32x9x9 -> 16x32x248x248, 32-point windows"}
+    del ws4
     # the other two passes (o4 as gradOutput): accGradParameters on the same descriptors,
     # updateGradInput on its own grid of disjoint gradInput windows
     bins, bouts, nbp = F.make_tile_grid(x4, o4, 9, 9, 32, F.FFT_UpdateGradInput)

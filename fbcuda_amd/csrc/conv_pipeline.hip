@@ -22,7 +22,14 @@
 //   3. inverseBinMajor:  C[bin][i][j] -> planes, gathering runs of SLOTS
 //      consecutive j per bin, inverse transform, crop on store.
 //
-// Spectra are unpacked (N/2+1 rows) so the contraction is a plain complex GEMM.
+// Spectral rows 0 and N/2 of a real plane are both Hermitian along kx, so their
+// 2 N complex values carry N complex worth of information; they travel as N
+// "virtual bins": v = x (0 < x < N/2) is row 0 at x, v = N/2 + x is row N/2 at x, and
+// v = 0 / v = N/2 hold the four real values (row 0 at 0 and N/2) / (row N/2 at 0 and
+// N/2) as (re, im) pairs.  The contraction is then a plain complex GEMM on N^2/2 bins;
+// only the two bins of real pairs multiply component by component instead (the product
+// rule of fbfft/FFTIteratedConvolution.cuh:161-186 with the unpacking done once, when
+// the forward transform stores the spectrum).
 //
 // All three passes are the same product P[i][j] = sum_k X[i][k] * op(Y[j][k]) with
 // the roles of MM-inl.cuh:188-196: forward (i, j, k) = (image, output plane, input
@@ -52,7 +59,7 @@ struct BMCfg {
   // transposed accesses (16 or more planes at the same bin) spread over the banks
   static constexpr int PSZ = (H + 1) * RS;
   static_assert((2 * PSZ) % 32 == 4 && PSZ % 2 == 0, "plane stride");
-  static constexpr int BINS = (H + 1) * N;
+  static constexpr int BINS = H * N;      // N virtual bins of rows 0 and N/2, then rows 1 .. N/2-1
 };
 
 // A family of planes indexed by (row, k).  Plain: plane (row, k) is the h x w window at
@@ -98,17 +105,44 @@ __device__ __forceinline__ PlaneWindow planeWindow(const PlaneSet& ps, int row, 
 }
 
 // ---- 1. planes -> S[bin][k][row] ----
-// PAIRS: every plane of the set passes windowMovesAsPairs() (8-byte words per row)
+// One operand of the product: its planes, where its spectra go, and how many
+// workgroups (row groups x Kp) transform it.
+struct ForwardJob {
+  PlaneSet ps;
+  float2* S;
+  int Rp, Kp;
+  float imSign;
+  int rowGroups;  // Rp / SLOTS
+};
+
+// Both operands of a pass in one launch: workgroups [0, a.rowGroups * a.Kp) transform
+// a's planes, the rest b's.  PAIRS_x: every plane of that set passes
+// windowMovesAsPairs() (8-byte words per row).
 template <int N, int PAIRS>
-__global__ __launch_bounds__(kT) void forwardBinMajor(PlaneSet ps, float2* S, int Rp, int Kp,
-                                                      float imSign) {
+__device__ __forceinline__ void forwardBinMajorBody(const ForwardJob& job, int wg, c32* lds);
+
+template <int N, int PAIRS_A, int PAIRS_B>
+__global__ __launch_bounds__(kT) void forwardBinMajor(ForwardJob a, ForwardJob b) {
+  __shared__ __align__(16) c32 lds[BMCfg<N>::SLOTS * BMCfg<N>::PSZ];
+  const int nA = a.rowGroups * a.Kp;
+  if ((int)blockIdx.x < nA)
+    forwardBinMajorBody<N, PAIRS_A>(a, blockIdx.x, lds);
+  else
+    forwardBinMajorBody<N, PAIRS_B>(b, blockIdx.x - nA, lds);
+}
+
+template <int N, int PAIRS>
+__device__ __forceinline__ void forwardBinMajorBody(const ForwardJob& job, int wg, c32* lds) {
   using C = BMCfg<N>;
   constexpr int H = C::H, T = C::T, SLOTS = C::SLOTS, RS = C::RS, PSZ = C::PSZ;
-  __shared__ __align__(16) c32 lds[SLOTS * PSZ];
+  const PlaneSet& ps = job.ps;
+  float2* S = job.S;
+  const int Rp = job.Rp, Kp = job.Kp;
+  const float imSign = job.imSign;
   const int t = threadIdx.x;
   const int s = t / T, l = t % T;
-  const int r0 = blockIdx.x * SLOTS;
-  const int k = blockIdx.y;
+  const int r0 = (wg % job.rowGroups) * SLOTS;
+  const int k = wg / job.rowGroups;
   const int row = r0 + s;
 
   c32 z0[H], z1[H];
@@ -132,23 +166,27 @@ __global__ __launch_bounds__(kT) void forwardBinMajor(PlaneSet ps, float2* S, in
   const c32* src = lds + sp * PSZ + bq;
   const long binStride = (long)Kp * Rp;
   float2* dst = S + (long)k * Rp + r0 + sp + bq * binStride;
-  auto put = [&](int bin, c32 v) __attribute__((always_inline)) {
-    v.y *= imSign;
-    dst[bin * binStride] = v;
-  };
-  // rows 0 and N/2 share packed row 0: F0[x] = (P[x] + conj P[N-x]) / 2,
-  // FH[x] = (P[x] - conj P[N-x]) / 2i
-  staticFor<2>([&](auto ee) {
-    constexpr int e = decltype(ee)::value;
-    const int x = bq + T * e;
-    const c32 a = src[T * e], m = lds[sp * PSZ + ((N - x) & (N - 1))];
-    put(T * e, c32{0.5f * (a.x + m.x), 0.5f * (a.y - m.y)});
-    put(H * N + T * e, c32{0.5f * (a.y + m.y), 0.5f * (m.x - a.x)});
-  });
+  auto put = [&](int bin, c32 v) __attribute__((always_inline)) { dst[bin * binStride] = v; };
+  // Packed row 0 holds P[x] = F0[x] + i FH[x]: F0[x] = (P[x] + conj P[N-x]) / 2,
+  // FH[x] = (P[x] - conj P[N-x]) / 2i.  Lane bq stores virtual bins bq (F0) and
+  // T + bq (FH); bq = 0 stores the real pairs (F0[0], F0[N/2]) and (FH[0], FH[N/2]),
+  // which no conjugation touches.
+  {
+    const c32 a = src[0], m = lds[sp * PSZ + (bq == 0 ? H : N - bq)];
+    c32 f0 = c32{0.5f * (a.x + m.x), 0.5f * (a.y - m.y) * imSign};
+    c32 fh = c32{0.5f * (a.y + m.y), 0.5f * (m.x - a.x) * imSign};
+    if (bq == 0) {
+      f0 = c32{a.x, m.x};
+      fh = c32{a.y, m.y};
+    }
+    put(0, f0);
+    put(T, fh);
+  }
   staticFor<H - 1>([&](auto rr) {
     constexpr int r = decltype(rr)::value + 1;
-    put(r * N, src[r * RS]);
-    put(r * N + T, src[r * RS + T]);
+    const c32 u = src[r * RS], v = src[r * RS + T];
+    put(r * N, c32{u.x, u.y * imSign});
+    put(r * N + T, c32{v.x, v.y * imSign});
   });
 }
 
@@ -184,17 +222,18 @@ __global__ __launch_bounds__(kT) void inverseBinMajor(const float2* Cs, int I, i
   }
   __syncthreads();
   c32* plane = lds + s * PSZ;
-  {  // pack rows 0 and H: Q = F0 + i*FH, real parts only at x = 0 (fbfft/FFT2D32.cuh:310-316)
-    c32* r0 = plane + 2 * l;
-    const c32* rH = r0 + H * RS;
-    float4 a = ldsLoad4(r0);
-    float4 c = ldsLoad4(rH);
-    float4 q = float4{a.x - c.y, a.y + c.x, a.z - c.w, a.w + c.z};
+  {  // virtual bins of row 0 back to the packed row: Q[x] = C0[x] + i CH[x],
+     // Q[N-x] = conj(C0[x]) + i conj(CH[x]); lane 0 sorts the four real values into
+     // Q[0] = (C0[0], CH[0]) and Q[N/2] = (C0[N/2], CH[N/2]).  The T lanes of a plane
+     // sit in one wave: all of them have read before any of them writes.
+    const c32 c0 = plane[l], cH = plane[T + l];
+    c32 q = c32{c0.x - cH.y, c0.y + cH.x}, qm = c32{c0.x + cH.y, cH.x - c0.y};
     if (l == 0) {
-      q.x = a.x;
-      q.y = c.x;
+      q = c32{c0.x, cH.x};
+      qm = c32{c0.y, cH.y};
     }
-    *reinterpret_cast<float4*>(r0) = q;
+    plane[l] = q;
+    plane[l == 0 ? H : N - l] = qm;
   }
   __syncthreads();
   rowPassInPlace<N, false>(plane, l);
@@ -202,6 +241,10 @@ __global__ __launch_bounds__(kT) void inverseBinMajor(const float2* Cs, int I, i
   c32 z0[H], z1[H];
   columnPassInverse<N>(plane, l, z0, z1);
   const int j = j0 + s;
+  // (Parking the cropped planes in LDS and writing them out as 16-byte runs - one
+  // contiguous stream for dense outputs, row quads for windows of a tiled image - was
+  // measured and is slower, 35.9 -> 36.6 us at configs[3] and 112 -> 131 us at
+  // configs[4]: the kernel waits on its own chain of phases, not on store requests.)
   if (j < out.K) {  // out.K: number of valid output planes along j
     const PlaneWindow win = planeWindow(out, i, j);
     storeColumnsWindow<N, ACC>(win.p, out.sy, out.sx, win.h, win.w, win.padL, win.padU, l, z0, z1,
@@ -218,6 +261,7 @@ struct GemmArgs {
   float2* C;        // [bins][I][Jp]
   int bins, I, Ip, Jp, Kp;
   int IT, JT;       // tiles per bin
+  int N;            // transform size: bins 0 and N/2 hold pairs of real values
   float invNorm;
 };
 
@@ -267,6 +311,9 @@ __global__ __launch_bounds__(kT, TI == 128 ? 3 : 4) void binGemmDirect(GemmArgs 
   const int i0 = (rem / g.JT) * TI, j0 = (rem % g.JT) * GJ2;
   const int rb = TI == 128 ? w : w % 2;  // 32-row block of this wave
   const int cb = TI == 128 ? 0 : w / 2;  // first 32-column block of this wave
+  // bins of real pairs: (ar br, ai bi) instead of a complex product; k1 and k3 hold them
+  const bool pairs = bin == 0 || 2 * bin == g.N;
+  const float cross = pairs ? 0.f : 1.f;
 
   const float2* Ab = g.A + (long)bin * g.Kp * g.Ip;
   const float2* Bb = g.B + (long)bin * g.Kp * g.Jp;
@@ -324,11 +371,11 @@ __global__ __launch_bounds__(kT, TI == 128 ? 3 : 4) void binGemmDirect(GemmArgs 
 #pragma unroll
     for (int s2 = 0; s2 < GK2 / 2; ++s2) {
       const float2 a = av[s2];
-      const float as = a.x + a.y;
+      const float as = __builtin_fmaf(cross, a.y, a.x);
 #pragma unroll
       for (int q = 0; q < NQ; ++q) {
         const float2 b = bv[s2][q];
-        const float nbs = -b.x - b.y, bd = b.x - b.y;
+        const float nbs = -b.x - b.y, bd = __builtin_fmaf(cross, b.x, -b.y);
         k1[q] = __builtin_amdgcn_mfma_f32_32x32x2f32(as, b.x, k1[q], 0, 0, 0);
         k2[q] = __builtin_amdgcn_mfma_f32_32x32x2f32(a.x, nbs, k2[q], 0, 0, 0);
         k3[q] = __builtin_amdgcn_mfma_f32_32x32x2f32(a.y, bd, k3[q], 0, 0, 0);
@@ -360,7 +407,106 @@ __global__ __launch_bounds__(kT, TI == 128 ? 3 : 4) void binGemmDirect(GemmArgs 
       const int i = i0 + 32 * rb + 8 * (v / 4) + 4 * h + v % 4;
       if (i < g.I)
         Cb[(long)i * g.Jp + j] =
-            float2{(k1[q][v] - k3[q][v]) * g.invNorm, (k1[q][v] + k2[q][v]) * g.invNorm};
+            pairs ? float2{k1[q][v] * g.invNorm, -k3[q][v] * g.invNorm}
+                  : float2{(k1[q][v] - k3[q][v]) * g.invNorm, (k1[q][v] + k2[q][v]) * g.invNorm};
+    }
+  }
+}
+
+// The same product with no LDS and no barriers: a wave owns one 32 x 32 sub-tile and
+// loads exactly the operand values its own MFMA lanes supply - lane (r, h) of
+// v_mfma_f32_32x32x2_f32 supplies row / column r at k = h, so one 8-byte load per lane
+// fetches k-rows 2s and 2s+1 of 32 consecutive rows (two 256-byte runs per wave
+// instruction).  Slices of 8 k ride a ring of three register sets, two in flight while
+// one is multiplied.  The four waves of a workgroup are the 2 x 2 sub-tiles of a
+// 64 x 64 tile: they re-read each other's operands out of the CU's vector cache,
+// nothing else ties them together.
+struct GemmSlice {
+  float2 a[GK2 / 2], b[GK2 / 2];
+};
+
+__global__ __launch_bounds__(kT, 4) void binGemmRegs(GemmArgs g) {
+  const int t = threadIdx.x;
+  const int lane = t % 64, w = t / 64;
+  const int r = lane % 32, h = lane / 32;
+  const int total = g.bins * g.IT * g.JT;
+  const int per = (total + 7) / 8;
+  const int logical = (blockIdx.x % 8) * per + blockIdx.x / 8;
+  if (logical >= total) return;
+  const int bin = logical / (g.IT * g.JT);
+  const int rem = logical % (g.IT * g.JT);
+  const int i0 = (rem / g.JT) * 64 + 32 * (w % 2), j0 = (rem % g.JT) * 64 + 32 * (w / 2);
+  if (i0 >= g.I || j0 >= g.Jp) return;  // sub-tile past the edge: nothing to compute
+  const bool pairs = bin == 0 || 2 * bin == g.N;  // bins of real pairs: (ar br, ai bi)
+  const float cross = pairs ? 0.f : 1.f;
+
+  // operand columns beyond the padded arrays are clamped (they feed accumulators that
+  // are never stored)
+  const float2* pa = g.A + ((long)bin * g.Kp + h) * g.Ip + min(i0 + r, g.Ip - 1);
+  const float2* pb = g.B + ((long)bin * g.Kp + h) * g.Jp + min(j0 + r, g.Jp - 1);
+  const long sa = 2L * g.Ip, sb = 2L * g.Jp;  // two k-rows
+
+  floatx16 k1, k2, k3;
+#pragma unroll
+  for (int v = 0; v < 16; ++v) k1[v] = k2[v] = k3[v] = 0.f;
+
+  const int slices = g.Kp / GK2;
+  auto fetch = [&](GemmSlice& s, int sl) __attribute__((always_inline)) {
+    const float2* qa = pa + (long)sl * (GK2 / 2) * sa;
+    const float2* qb = pb + (long)sl * (GK2 / 2) * sb;
+#pragma unroll
+    for (int u = 0; u < GK2 / 2; ++u) {
+      s.a[u] = qa[u * sa];
+      s.b[u] = qb[u * sb];
+    }
+  };
+  // a conj(b) = (k1 - k3) + i (k1 + k2) with k1 = (ar + ai) br, k2 = -ar (br + bi),
+  // k3 = ai (br - bi)
+  auto multiply = [&](const GemmSlice& s) __attribute__((always_inline)) {
+#pragma unroll
+    for (int u = 0; u < GK2 / 2; ++u) {
+      const float2 a = s.a[u], b = s.b[u];
+      k1 = __builtin_amdgcn_mfma_f32_32x32x2f32(__builtin_fmaf(cross, a.y, a.x), b.x, k1, 0, 0, 0);
+      k2 = __builtin_amdgcn_mfma_f32_32x32x2f32(a.x, -b.x - b.y, k2, 0, 0, 0);
+      k3 = __builtin_amdgcn_mfma_f32_32x32x2f32(a.y, __builtin_fmaf(cross, b.x, -b.y), k3, 0, 0, 0);
+    }
+  };
+  GemmSlice s0, s1, s2;
+  fetch(s0, 0);
+  fetch(s1, min(1, slices - 1));
+  int sl = 0;
+  // the scheduling barriers keep each slice's loads ahead of the products of the slice
+  // two before it; left alone the compiler sinks the loads below the products and then
+  // waits for all of them at the top of the loop
+  for (; sl + 3 <= slices; sl += 3) {
+    fetch(s2, min(sl + 2, slices - 1));
+    __builtin_amdgcn_sched_barrier(0);
+    multiply(s0);
+    __builtin_amdgcn_sched_barrier(0);
+    fetch(s0, min(sl + 3, slices - 1));
+    __builtin_amdgcn_sched_barrier(0);
+    multiply(s1);
+    __builtin_amdgcn_sched_barrier(0);
+    fetch(s1, min(sl + 4, slices - 1));
+    __builtin_amdgcn_sched_barrier(0);
+    multiply(s2);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  if (sl < slices) {
+    multiply(s0);
+    if (sl + 1 < slices) multiply(s1);
+  }
+
+  float2* Cb = g.C + (long)bin * g.I * g.Jp;
+  const int j = j0 + r;
+  if (j < g.Jp) {
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      const int i = i0 + 8 * (v / 4) + 4 * h + v % 4;
+      if (i < g.I)
+        Cb[(long)i * g.Jp + j] =
+            pairs ? float2{k1[v] * g.invNorm, -k3[v] * g.invNorm}
+                  : float2{(k1[v] - k3[v]) * g.invNorm, (k1[v] + k2[v]) * g.invNorm};
     }
   }
 }
@@ -405,23 +551,28 @@ int runPipeline(PlaneSet x, PlaneSet y, PlaneSet out, bool conjY, float scale, b
   float2* SB = SA + (size_t)bins * Kp * Ip;
   float2* SC = SB + (size_t)bins * Kp * Jp;
 
-  auto forward = [&](const PlaneSet& p, float2* S, int Rp, float sign) {
-    // every window of the set starts on an 8-byte boundary with an even width and pad
-    const bool pairs = windowMovesAsPairs(p.base, p.sy, p.sx, p.w, p.padL0) && p.sRow % 2 == 0 &&
-                       p.sK % 2 == 0 &&
-                       (!p.tiled || ((p.stepX | p.orgX | p.winW) & 1) == 0);
-    if (pairs)
-      forwardBinMajor<N, 1><<<dim3(Rp / SL, Kp), dim3(kT), 0, s>>>(p, S, Rp, Kp, sign);
-    else
-      forwardBinMajor<N, 0><<<dim3(Rp / SL, Kp), dim3(kT), 0, s>>>(p, S, Rp, Kp, sign);
+  // every window of a set starts on an 8-byte boundary with an even width and pad
+  auto movesAsPairs = [](const PlaneSet& p) {
+    return windowMovesAsPairs(p.base, p.sy, p.sx, p.w, p.padL0) && p.sRow % 2 == 0 &&
+           p.sK % 2 == 0 && (!p.tiled || ((p.stepX | p.orgX | p.winW) & 1) == 0);
   };
-  forward(x, SA, Ip, xSign);
-  forward(y, SB, Jp, ySign);
+  const ForwardJob ja{x, SA, Ip, Kp, xSign, Ip / SL}, jb{y, SB, Jp, Kp, ySign, Jp / SL};
+  const dim3 fgrid((unsigned)(ja.rowGroups + jb.rowGroups) * Kp);
+  const bool pa = movesAsPairs(x), pb = movesAsPairs(y);
+  if (pa && pb)
+    forwardBinMajor<N, 1, 1><<<fgrid, dim3(kT), 0, s>>>(ja, jb);
+  else if (pa)
+    forwardBinMajor<N, 1, 0><<<fgrid, dim3(kT), 0, s>>>(ja, jb);
+  else if (pb)
+    forwardBinMajor<N, 0, 1><<<fgrid, dim3(kT), 0, s>>>(ja, jb);
+  else
+    forwardBinMajor<N, 0, 0><<<fgrid, dim3(kT), 0, s>>>(ja, jb);
   GemmArgs g;
   g.A = SA;
   g.B = SB;
   g.C = SC;
   g.bins = bins;
+  g.N = N;
   g.I = I;
   g.Ip = Ip;
   g.Jp = Jp;
@@ -432,7 +583,13 @@ int runPipeline(PlaneSet x, PlaneSet y, PlaneSet out, bool conjY, float scale, b
   // chip with fewer than eight workgroups per CU to balance (measured equal or
   // faster there: 84 -> 62 us for 64 x 192 x 128 per bin, 77 -> 69 us for 128 x 64 x 192)
   const bool small = roundUp(I, 64) < roundUp(I, GI) || (long)bins * ceilDiv(I, GI) * g.JT < 8 * 256;
-  if (small) {
+  // Up to 32 columns the LDS kernels' 64-column tiles would be half empty; the register
+  // kernel drops its idle sub-tiles (configs[4], 1936 x 32 x 32 per bin: 146 -> 139 us.
+  // At configs[3], 128 x 192 x 64 per bin, it is the slower one: 64 against 58 us.)
+  if (Jp <= 32) {
+    g.IT = ceilDiv(I, 64);
+    binGemmRegs<<<dim3(roundUp(bins * g.IT * g.JT, 8)), dim3(kT), 0, s>>>(g);
+  } else if (small) {
     g.IT = ceilDiv(I, 64);
     binGemmDirect<64><<<dim3(roundUp(bins * g.IT * g.JT, 8)), dim3(kT), 0, s>>>(g);
   } else {
