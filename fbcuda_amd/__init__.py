@@ -46,7 +46,8 @@ _lib = None
 # every symbol include/fbfft_amd.h declares
 EXPORTS = (
     "fbfft_r2c_1d", "fbfft_c2r_1d", "fbfft_r2c_2d", "fbfft_c2c_2d_pass2", "fbfft_c2r_2d",
-    "fbfft_c2c_2d_inverse_pass1", "fbfft_transpose_mm", "fbfft_transpose_mm_packed", "fbfft_iterated_conv", "fbfft_make_tiles",
+    "fbfft_c2c_2d_inverse_pass1", "fbfft_transpose_mm", "fbfft_transpose_mm_packed", "fbfft_iterated_conv", "fbfft_iterated_conv_ex",
+    "fbfft_make_tiles",
     "fbfft_make_tiles_for_pass",
     "fbfft_conv_workspace", "fbfft_conv_workspace_image", "fbfft_conv_fprop_workspace", "fbfft_conv_fprop", "fbfft_conv_bprop",
     "fbfft_conv_accgrad", "fbfft_conv_fprop_static", "fbfft_error_string",
@@ -76,6 +77,8 @@ def lib():
         L.fbfft_transpose_mm_packed.argtypes = L.fbfft_transpose_mm.argtypes
         L.fbfft_iterated_conv.argtypes = [ctypes.c_int, vp, vp, tp, ctypes.c_int, ctypes.c_float,
                                           ctypes.c_int, ctypes.c_size_t, vp]
+        L.fbfft_iterated_conv_ex.argtypes = [ctypes.c_int, vp, vp, tp, ctypes.c_int, ctypes.c_float,
+                                             ctypes.c_int, ctypes.c_size_t, ctypes.c_uint, vp]
         L.fbfft_make_tiles.argtypes = [tp, tp, ctypes.c_int, ctypes.c_int, ctypes.c_int, vp, vp,
                                        ctypes.c_size_t]
         L.fbfft_make_tiles.restype = ctypes.c_size_t
@@ -229,16 +232,22 @@ def make_tile_grid(input, output, kH, kW, fftSize, pass_=FFT_UpdateOutput):
     return up(a), up(b), n
 
 
+DETERMINISTIC = 1
+
+
 def FFTIteratedConvolution(fftSize, ins, outs, weight, pass_, scale, batchSize, numTiles,
-                           stream=None):
+                           stream=None, deterministic=False):
     """detail::FFTIteratedConvolution<fftSize> (fbfft/FFTIteratedConvolution.cuh:624-755).
 
     ins / outs: device uint8 tensors from make_tiles.  Returns True if launched.
+    deterministic: FFT_AccGradParameters reduces in the reference's fixed order (one
+    workgroup per plane group, no atomic adds): reproducible bit for bit, much slower.
     """
     _on_gpu(ins, outs, weight)
-    rc = lib().fbfft_iterated_conv(fftSize, ctypes.c_void_p(ins.data_ptr()),
-                                   ctypes.c_void_p(outs.data_ptr()), view(weight), int(pass_),
-                                   float(scale), int(batchSize), int(numTiles), _stream(stream))
+    rc = lib().fbfft_iterated_conv_ex(fftSize, ctypes.c_void_p(ins.data_ptr()),
+                                      ctypes.c_void_p(outs.data_ptr()), view(weight), int(pass_),
+                                      float(scale), int(batchSize), int(numTiles),
+                                      DETERMINISTIC if deterministic else 0, _stream(stream))
     if rc < 0:
         raise RuntimeError("fbfft_iterated_conv: %s" % error_string(-rc))
     return rc == 1

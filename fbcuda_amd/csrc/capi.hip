@@ -421,10 +421,19 @@ extern "C" size_t fbfft_make_tiles(const fbfft_tensor* input, const fbfft_tensor
 extern "C" int fbfft_iterated_conv(int fftSize, const fbfft_tile* ins, const fbfft_tile* outs,
                                    const fbfft_tensor* weight, int pass, float scale,
                                    int batchSize, size_t numTiles, fbfft_stream_t stream) {
+  return fbfft_iterated_conv_ex(fftSize, ins, outs, weight, pass, scale, batchSize, numTiles, 0,
+                                stream);
+}
+
+extern "C" int fbfft_iterated_conv_ex(int fftSize, const fbfft_tile* ins, const fbfft_tile* outs,
+                                      const fbfft_tensor* weight, int pass, float scale,
+                                      int batchSize, size_t numTiles, unsigned flags,
+                                      fbfft_stream_t stream) {
   if (!okTensor(weight, 4) || !ins || !outs) return 0;
+  if (flags & ~(unsigned)FBFFT_DETERMINISTIC) return 0;
   // a filter larger than the transform has no circular-convolution meaning; the
   // windowed loader would silently drop its rows / columns beyond fftSize
   if (weight->size[2] > fftSize || weight->size[3] > fftSize) return 0;
   return launchIteratedConv(fftSize, ins, outs, weight->data, weight->stride, weight->size, pass,
-                            scale, batchSize, numTiles, stream);
+                            scale, batchSize, numTiles, (flags & FBFFT_DETERMINISTIC) != 0, stream);
 }

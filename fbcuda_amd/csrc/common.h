@@ -66,7 +66,7 @@ int launchTransposeMMPacked(const float* A, long a0, long a1, const float* B, lo
 
 int launchIteratedConv(int N, const fbfft_tile* ins, const fbfft_tile* outs, float* weight,
                        const int* wStride, const int* wSize, int pass, float scale, int batch,
-                       size_t numTiles, hipStream_t s);
+                       size_t numTiles, bool deterministic, hipStream_t s);
 
 // mode 0/1: forward pass 1/2, mode 2/3: inverse pass 1/2 of the two-call 64/128 forms
 int launchTwoPass(int N, int mode, float* src, long s0, long s1, long s2, float* dst, long d0,

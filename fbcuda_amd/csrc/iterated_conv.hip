@@ -349,7 +349,7 @@ __global__ void zeroWeight(ConvArgs a) {
 }
 
 template <int N>
-int launchPass(int pass, const ConvArgs& a, hipStream_t s) {
+int launchPass(int pass, const ConvArgs& a, bool deterministic, hipStream_t s) {
   using C = ConvCfg<N>;
   const int Cout = a.wn[0], Cin = a.wn[1];
   if (pass == FBFFT_UPDATE_OUTPUT) {
@@ -368,7 +368,11 @@ int launchPass(int pass, const ConvArgs& a, hipStream_t s) {
     ConvArgs b = a;
     const int groups = ceilDiv(Cout, C::FO) * ceilDiv(Cin, C::BN);
     const int steps = a.numTiles * a.batch;
-    b.splits = std::max(1, std::min(ceilDiv(512, groups), ceilDiv(steps, 2 * C::SPI)));
+    // deterministic: the reference's schedule, one workgroup per plane group over the
+    // whole reduction in a fixed order, no atomics (and most of the chip idle)
+    b.splits = deterministic
+                   ? 1
+                   : std::max(1, std::min(ceilDiv(512, groups), ceilDiv(steps, 2 * C::SPI)));
     if (b.splits > 1) {
       const long total = (long)a.wn[0] * a.wn[1] * a.wn[2] * a.wn[3];
       zeroWeight<<<dim3((unsigned)std::min<long>((total + 255) / 256, 4096)), 256, 0, s>>>(b);
@@ -384,7 +388,7 @@ int launchPass(int pass, const ConvArgs& a, hipStream_t s) {
 // returns 1 launched, 0 nothing matched, -FBFFT_HIP_ERROR on launch failure
 int launchIteratedConv(int N, const fbfft_tile* ins, const fbfft_tile* outs, float* weight,
                        const int* wStride, const int* wSize, int pass, float scale, int batch,
-                       size_t numTiles, hipStream_t s) {
+                       size_t numTiles, bool deterministic, hipStream_t s) {
   if (!(N == 8 || N == 16 || N == 32)) return 0;
   if (pass < 0 || pass > 2) return 0;
   ConvArgs a;
@@ -400,8 +404,9 @@ int launchIteratedConv(int N, const fbfft_tile* ins, const fbfft_tile* outs, flo
   a.splits = 1;
   a.scale = scale;
   if (batch <= 0 || numTiles == 0 || wSize[0] <= 0 || wSize[1] <= 0) return 1;  // nothing to do
-  int rc = N == 8 ? launchPass<8>(pass, a, s) : N == 16 ? launchPass<16>(pass, a, s)
-                                                        : launchPass<32>(pass, a, s);
+  int rc = N == 8    ? launchPass<8>(pass, a, deterministic, s)
+           : N == 16 ? launchPass<16>(pass, a, deterministic, s)
+                     : launchPass<32>(pass, a, deterministic, s);
   return rc == FBFFT_SUCCESS ? 1 : -rc;
 }
 

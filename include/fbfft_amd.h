@@ -154,6 +154,19 @@ int fbfft_iterated_conv(int fftSize, const fbfft_tile* ins, const fbfft_tile* ou
                         const fbfft_tensor* weight, int pass, float scale, int batchSize,
                         size_t numTiles, fbfft_stream_t stream);
 
+/* The same with flags.  FBFFT_DETERMINISTIC: FBFFT_ACC_GRAD_PARAMETERS runs the
+ * reference's schedule - one workgroup per group of weight planes walks the whole
+ * (tile, image) reduction in a fixed order (fbfft/FFTIteratedConvolution.cuh:
+ * 600-613), no atomic adds - so the result is bit-for-bit reproducible from run to
+ * run, at the price of leaving most of the chip idle (configs[4]: 10.5 ms instead of
+ * 0.63 ms).  fbfft_conv_accgrad on the whole image is both reproducible and fast; it
+ * needs a workspace.  The other passes are reproducible either way.  Unknown flag
+ * bits return 0. */
+#define FBFFT_DETERMINISTIC 1u
+int fbfft_iterated_conv_ex(int fftSize, const fbfft_tile* ins, const fbfft_tile* outs,
+                           const fbfft_tensor* weight, int pass, float scale, int batchSize,
+                           size_t numTiles, unsigned flags, fbfft_stream_t stream);
+
 /* Host-side builder of the tile descriptors FFTIteratedConvolution consumes; the
  * reference leaves this to its external caller (fbfft/FFTIteratedConvolution.cuh:
  * 71-88 declares the descriptor, :113-114 consumes ins[tile] / outs[tile]).

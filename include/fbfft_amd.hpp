@@ -455,15 +455,19 @@ typedef struct _FFTConvolutionPassFFI {
   int pass;
 } FFTConvolutionPassFFI;
 
-// ins / outs: device pointers to numTiles descriptors
+// ins / outs: device pointers to numTiles descriptors.  deterministic (not in the
+// reference's signature): FFT_AccGradParameters reduces in the reference's fixed order,
+// reproducible bit for bit and much slower; see fbfft_iterated_conv_ex.
 template <int FFTSize>
 bool FFTIteratedConvolution(TiledDeviceTensor<float, 4>* ins, TiledDeviceTensor<float, 4>* outs,
                             const DeviceTensor<float, 4> weight, FFTConvolutionPassFFI pass,
-                            float scale, int batchSize, size_t numTiles, fbfft_stream_t s) {
+                            float scale, int batchSize, size_t numTiles, fbfft_stream_t s,
+                            bool deterministic = false) {
   fbfft_tensor w = fbfft_amd_detail::describe(weight);
-  return fbfft_iterated_conv(FFTSize, reinterpret_cast<const fbfft_tile*>(ins),
-                             reinterpret_cast<const fbfft_tile*>(outs), &w, pass.pass, scale,
-                             batchSize, numTiles, s) == 1;
+  return fbfft_iterated_conv_ex(FFTSize, reinterpret_cast<const fbfft_tile*>(ins),
+                                reinterpret_cast<const fbfft_tile*>(outs), &w, pass.pass, scale,
+                                batchSize, numTiles, deterministic ? FBFFT_DETERMINISTIC : 0u,
+                                s) == 1;
 }
 
 // Host-side tile grid for FFTIteratedConvolution<FFTSize>: fills ins / outs (host

@@ -206,3 +206,50 @@ def test_random_tilings(oracle, seed):
     assert F.FFTIteratedConvolution(N, bins, bouts, w, F.FFT_UpdateGradInput, 1.0, Nb, n3), tag
     torch.cuda.synchronize()
     assert rel(gin.cpu().numpy(), oracle.corr2d_grad_input(g.cpu().numpy(), wh, H, W)) < TOL_CONV, tag
+
+
+def test_deterministic_weight_gradient_is_reproducible(oracle):
+    """FBFFT_DETERMINISTIC: accGradParameters in the reference's fixed order gives the same
+    bits on every run (the default schedule adds range partials atomically, in any order)
+    and the same values as the fp64 gradient."""
+    N, k, H, W, Nb, Cin, Cout = 16, 5, 60, 52, 6, 5, 7
+    d = dev()
+    x = synth.uniform((Nb, Cin, H, W), seed=70, device=d)
+    g = synth.normal((Nb, Cout, H - k + 1, W - k + 1), seed=71, device=d)
+    ins, outs, n = F.make_tile_grid(x, g, k, k, N)
+    runs = []
+    for _ in range(3):
+        gw = torch.full((Cout, Cin, k, k), float("nan"), device=d)
+        assert F.FFTIteratedConvolution(N, ins, outs, gw, F.FFT_AccGradParameters, 0.5, Nb, n,
+                                        deterministic=True)
+        torch.cuda.synchronize()
+        runs.append(gw.cpu().numpy())
+    assert np.array_equal(runs[0], runs[1]) and np.array_equal(runs[0], runs[2])
+    want = 0.5 * oracle.corr2d_grad_weight(x.cpu().numpy(), g.cpu().numpy(), k, k)
+    assert rel(runs[0], want) < TOL_CONV
+    # the default schedule agrees to rounding
+    gw = torch.full((Cout, Cin, k, k), float("nan"), device=d)
+    assert F.FFTIteratedConvolution(N, ins, outs, gw, F.FFT_AccGradParameters, 0.5, Nb, n)
+    torch.cuda.synchronize()
+    assert rel(gw.cpu().numpy(), runs[0]) < TOL_CONV
+    # unknown flag bits: not launched
+    rc = F.lib().fbfft_iterated_conv_ex(N, ins.data_ptr(), outs.data_ptr(), F.view(gw), 2, 0.5, Nb, n, 6,
+                                        None)
+    assert rc == 0
+
+
+def test_layer_weight_gradient_is_reproducible():
+    """fbfft_conv_accgrad on a tiled image: a fixed reduction order inside the contraction,
+    no atomics - the same bits on every run."""
+    N, k, H, W, Nb, Cin, Cout = 32, 5, 80, 71, 4, 6, 5
+    d = dev()
+    x = synth.uniform((Nb, Cin, H, W), seed=72, device=d)
+    g = synth.normal((Nb, Cout, H - k + 1, W - k + 1), seed=73, device=d)
+    ws = torch.empty(F.conv_workspace_image(2, Nb, Cin, Cout, H, W, k, k, N), dtype=torch.uint8, device=d)
+    runs = []
+    for _ in range(3):
+        gw = torch.full((Cout, Cin, k, k), float("nan"), device=d)
+        assert F.conv_accgrad(x, g, gw, N, ws) == F.Success
+        torch.cuda.synchronize()
+        runs.append(gw.cpu().numpy())
+    assert np.array_equal(runs[0], runs[1]) and np.array_equal(runs[0], runs[2])
