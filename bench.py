@@ -236,7 +236,17 @@ def conv_extras(F, synth, torch, dev, extra):
     extra["transposeMM_configs3_us"] = round(t * 1e6, 1)
     extra["transposeMM_configs3_TFLOPs"] = round(6.845e9 / t / 1e12, 1)
     extra["transposeMM_configs3_frac_of_fp32_mfma_peak"] = round(6.845e9 / t / 157.3e12, 4)
-    del A, Bm, C, x, w, out, ws
+    # the kernel issues three real products per complex one: 6 flop per multiply-add
+    extra["transposeMM_configs3_frac_issued"] = round(6.845e9 * 0.75 / t / 157.3e12, 4)
+    del A, Bm, C
+    # the same contraction on packed spectra (16 rows per plane instead of 17)
+    Ap = synth.normal((128, 64, 16, 32, 2), seed=30, device=dev)
+    Bp = synth.normal((192, 64, 16, 32, 2), seed=31, device=dev)
+    Cp = torch.empty((128, 192, 16, 32, 2), device=dev)
+    mmp = prepared("fbfft_transpose_mm_packed", F, Ap, Bp, Cp, 0, 1, 0, ctypes.c_float(1.0 / 1024))
+    _, t = timed(mmp, 200, 200, torch)
+    extra["transposeMM_packed_configs3_us"] = round(t * 1e6, 1)
+    del Ap, Bp, Cp, x, w, out, ws
     # a 64-point layer (plane-major spectra through transposeMM): 32x32x60x60 * 64x32x5x5
     x6 = synth.normal((32, 32, 60, 60), seed=50, device=dev)
     w6 = synth.normal((64, 32, 5, 5), seed=51, std=0.02, device=dev)
@@ -487,6 +497,13 @@ def main():
         # round-trip sanity on the benchmark tensors themselves
         err = float((back / (N * N) - x).double().norm() / x.double().norm())
         extra["roundtrip_rel_l2"] = err
+        # packed spectra of configs[1]: [B][16][32][2], 8192 bytes per plane
+        sp = torch.empty((B, N // 2, N, 2), device=dev)
+        _, lp = timed(prepared("fbfft_r2c_2d", F, x, sp, 0, 0), args.steps, args.warmup, torch)
+        _, lq = timed(prepared("fbfft_c2r_2d", F, sp, back, 0, 0), args.steps, args.warmup, torch)
+        extra["r2c_32x32_packed_b16384_GBps"] = round(B * 8192 / lp / 1e9, 1)
+        extra["c2r_32x32_packed_b16384_GBps"] = round(B * 8192 / lq / 1e9, 1)
+        del sp
         for n2, b2 in ((16, 262144), (8, 1048576), (64, 16384), (128, 4096)):
             x2 = synth.normal((b2, n2, n2), seed=2 + n2.bit_length() - 1, device=dev)
             s2 = torch.empty((b2, n2 // 2 + 1, n2, 2), device=dev)

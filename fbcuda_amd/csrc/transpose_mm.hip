@@ -166,20 +166,12 @@ __device__ __forceinline__ void stashSlice(float* re, float* im, const Fetch& f,
   }
 }
 
+// one workgroup's share: work item `logical` of a (PACKED0: of the packed row 0 of a)
 template <bool VEC4, bool PACKED0>
-__global__ __launch_bounds__(THREADS) void transposeMMKernel(MMArgs a) {
-  __shared__ __align__(8) float lds[LDS_FLOATS];  // two slice buffers; later the C staging area
+__device__ __forceinline__ void transposeMMBody(const MMArgs& a, int logical, float* lds) {
   const int t = threadIdx.x;
   const int lane = t % 64, w = t / 64;
-  // Workgroups are dealt round-robin to the 8 XCDs, each with its own L2.  Give
-  // every XCD a contiguous range of logical ids, ordered bin-chunk first, so that
-  // the tiles that re-read the same lines of A and B (and the two chunks that
-  // share a 128-byte line) meet in one L2.
   const int tilesJ = (a.J + TJ - 1) / TJ, tilesI = (a.I + TI - 1) / TI;
-  const int total = a.chunks * tilesI * tilesJ;
-  const int per = (total + 7) / 8;
-  const int logical = (blockIdx.x % 8) * per + blockIdx.x / 8;
-  if (logical >= total) return;
   const int x0 = (logical / (tilesI * tilesJ)) * (PACKED0 ? XB / 2 : XB);
   const int rem = logical % (tilesI * tilesJ);
   // PACKED0: the waves holding the real pairs of x = 0 multiply component by component
@@ -331,14 +323,49 @@ __global__ __launch_bounds__(THREADS) void transposeMMKernel(MMArgs a) {
     }
 }
 
-}  // namespace
+inline int workItems(const MMArgs& a) {
+  return a.chunks * ((a.J + TJ - 1) / TJ) * ((a.I + TI - 1) / TI);
+}
 
-// A, B, C: complex-as-float views collapsed to [d0][d1][xy][2] with unit xy
-// stride; s0/s1 are the float strides of the first two dimensions.
-int launchTransposeMM(const float* A, long a0, long a1, const float* B, long b0, long b1, float* C,
-                      long c0, long c1, int I, int J, int K, int XY, bool conjA, bool conjB,
-                      bool accumulate, float invNorm, hipStream_t s) {
-  if (I <= 0 || J <= 0 || XY <= 0) return FBFFT_SUCCESS;
+// Workgroups are dealt round-robin to the 8 XCDs, each with its own L2.  Every XCD
+// gets a contiguous range of logical ids, ordered bin-chunk first, so that the tiles
+// that re-read the same lines of A and B (and the two chunks that share a 128-byte
+// line) meet in one L2.
+__device__ __forceinline__ int logicalWorkItem(int total) {
+  const int per = (total + 7) / 8;
+  return (blockIdx.x % 8) * per + blockIdx.x / 8;
+}
+
+template <bool VEC4>
+__global__ __launch_bounds__(THREADS) void transposeMMKernel(MMArgs a, int total) {
+  __shared__ __align__(8) float lds[LDS_FLOATS];  // two slice buffers; later the C staging area
+  const int logical = logicalWorkItem(total);
+  if (logical < total) transposeMMBody<VEC4, false>(a, logical, lds);
+}
+
+// Packed spectra in one launch: work items [0, totalMain) are the plain bins of rows
+// 1 .. N/2-1, the rest the chunks of packed row 0 - a handful of workgroups that would
+// leave most of the chip idle in a launch of their own.
+template <bool VEC4>
+__global__ __launch_bounds__(THREADS) void transposeMMPackedKernel(MMArgs mainRows, int totalMain,
+                                                                   MMArgs row0, int totalRow0) {
+  __shared__ __align__(8) float lds[LDS_FLOATS];
+  // every XCD takes its share of the (slower) row-0 items first, then its range of
+  // plain items
+  const int perRow0 = (totalRow0 + 7) / 8, perMain = (totalMain + 7) / 8;
+  const int xcd = blockIdx.x % 8, slot = blockIdx.x / 8;
+  if (slot < perRow0) {
+    const int item = xcd * perRow0 + slot;
+    if (item < totalRow0) transposeMMBody<false, true>(row0, item, lds);
+  } else {
+    const int item = xcd * perMain + slot - perRow0;
+    if (slot - perRow0 < perMain && item < totalMain) transposeMMBody<VEC4, false>(mainRows, item, lds);
+  }
+}
+
+MMArgs makeArgs(const float* A, long a0, long a1, const float* B, long b0, long b1, float* C,
+                long c0, long c1, int I, int J, int K, int XY, bool conjA, bool conjB,
+                bool accumulate, float invNorm, int chunks) {
   MMArgs m;
   m.A = A;
   m.B = B;
@@ -358,50 +385,52 @@ int launchTransposeMM(const float* A, long a0, long a1, const float* B, long b0,
   m.bSign = conjB ? -1.f : 1.f;
   m.invNorm = invNorm;
   m.accumulate = accumulate ? 1 : 0;
-  m.chunks = ceilDiv(XY, XB);
-  const int total = m.chunks * ceilDiv(J, TJ) * ceilDiv(I, TI);
+  m.chunks = chunks;
+  return m;
+}
+
+bool movesAsFloat4(const float* A, long a0, long a1, const float* B, long b0, long b1, int XY) {
+  return aligned(A, 16) && aligned(B, 16) && a0 % 4 == 0 && a1 % 4 == 0 && b0 % 4 == 0 &&
+         b1 % 4 == 0 && XY % 2 == 0;
+}
+
+}  // namespace
+
+// A, B, C: complex-as-float views collapsed to [d0][d1][xy][2] with unit xy
+// stride; s0/s1 are the float strides of the first two dimensions.
+int launchTransposeMM(const float* A, long a0, long a1, const float* B, long b0, long b1, float* C,
+                      long c0, long c1, int I, int J, int K, int XY, bool conjA, bool conjB,
+                      bool accumulate, float invNorm, hipStream_t s) {
+  if (I <= 0 || J <= 0 || XY <= 0) return FBFFT_SUCCESS;
+  const MMArgs m = makeArgs(A, a0, a1, B, b0, b1, C, c0, c1, I, J, K, XY, conjA, conjB, accumulate,
+                            invNorm, ceilDiv(XY, XB));
+  const int total = workItems(m);
   dim3 grid((total + 7) / 8 * 8), block(THREADS);
-  const bool vec4 = aligned(A, 16) && aligned(B, 16) && a0 % 4 == 0 && a1 % 4 == 0 &&
-                    b0 % 4 == 0 && b1 % 4 == 0 && XY % 2 == 0;
-  if (vec4)
-    transposeMMKernel<true, false><<<grid, block, 0, s>>>(m);
+  if (movesAsFloat4(A, a0, a1, B, b0, b1, XY))
+    transposeMMKernel<true><<<grid, block, 0, s>>>(m, total);
   else
-    transposeMMKernel<false, false><<<grid, block, 0, s>>>(m);
+    transposeMMKernel<false><<<grid, block, 0, s>>>(m, total);
   return launchStatus();
 }
 
 // The same contraction on packed spectra [d0][d1][N/2][N][2]: rows 1 .. N/2-1 as
-// plain bins, row 0 by the unpack / multiply / re-pack rule.
+// plain bins, row 0 by the unpack / multiply / re-pack rule, all in one launch.
 int launchTransposeMMPacked(const float* A, long a0, long a1, const float* B, long b0, long b1,
                             float* C, long c0, long c1, int I, int J, int K, int N, bool conjA,
                             bool conjB, bool accumulate, float invNorm, hipStream_t s) {
   if (I <= 0 || J <= 0) return FBFFT_SUCCESS;
-  if (N > 2) {
-    const int rc = launchTransposeMM(A + 2 * N, a0, a1, B + 2 * N, b0, b1, C + 2 * N, c0, c1, I, J,
-                                     K, (N / 2 - 1) * N, conjA, conjB, accumulate, invNorm, s);
-    if (rc != FBFFT_SUCCESS) return rc;
-  }
-  MMArgs m;
-  m.A = A;
-  m.B = B;
-  m.C = C;
-  m.I = I;
-  m.J = J;
-  m.K = K;
-  m.XY = N;
-  m.aRow = conjA ? a1 : a0;
-  m.aK = conjA ? a0 : a1;
-  m.bK = conjB ? b1 : b0;
-  m.bCol = conjB ? b0 : b1;
-  m.cRow = c0;
-  m.cCol = c1;
-  m.aSign = conjA ? -1.f : 1.f;
-  m.bSign = conjB ? -1.f : 1.f;
-  m.invNorm = invNorm;
-  m.accumulate = accumulate ? 1 : 0;
-  m.chunks = N / XB;  // four x per workgroup, x < N/2
-  const int total = m.chunks * ceilDiv(J, TJ) * ceilDiv(I, TI);
-  transposeMMKernel<false, true><<<dim3((total + 7) / 8 * 8), dim3(THREADS), 0, s>>>(m);
+  const int XY = (N / 2 - 1) * N;
+  const MMArgs mainRows = makeArgs(A + 2 * N, a0, a1, B + 2 * N, b0, b1, C + 2 * N, c0, c1, I, J, K,
+                                   XY, conjA, conjB, accumulate, invNorm, ceilDiv(XY, XB));
+  // four x per workgroup, x < N/2
+  const MMArgs row0 = makeArgs(A, a0, a1, B, b0, b1, C, c0, c1, I, J, K, N, conjA, conjB,
+                               accumulate, invNorm, N / XB);
+  const int totalMain = workItems(mainRows), totalRow0 = workItems(row0);
+  dim3 grid(((totalMain + 7) / 8 + (totalRow0 + 7) / 8) * 8), block(THREADS);
+  if (movesAsFloat4(A + 2 * N, a0, a1, B + 2 * N, b0, b1, XY))
+    transposeMMPackedKernel<true><<<grid, block, 0, s>>>(mainRows, totalMain, row0, totalRow0);
+  else
+    transposeMMPackedKernel<false><<<grid, block, 0, s>>>(mainRows, totalMain, row0, totalRow0);
   return launchStatus();
 }
 

@@ -361,3 +361,16 @@ def test_conv_layer_random_shapes(oracle, seed):
     assert rel(out.cpu().numpy(), oracle.corr2d_valid(xh, wh)) < TOL_CONV, tag
     assert rel(gi.cpu().numpy(), oracle.corr2d_grad_input(gh, wh, H, W)) < TOL_CONV, tag
     assert rel(gw.cpu().numpy(), 2.0 * oracle.corr2d_grad_weight(xh, gh, kH, kW)) < TOL_CONV, tag
+
+
+@pytest.mark.parametrize("Cin", [5, 8, 12, 24, 40])
+def test_conv_fprop_many_full_tiles(oracle, Cin):
+    """512 x 512 outputs per bin in 8-point transforms: more 64 x 64 tiles of the contraction
+    than workgroups resident at once, so every workgroup walks several tiles; the reduction
+    lengths give one, two, three and five k-slices per tile."""
+    N, H, k, Bn, Cout = 8, 8, 3, 512, 512
+    x = synth.normal((Bn, Cin, H, H), seed=80).numpy()
+    w = synth.normal((Cout, Cin, k, k), seed=81, std=0.1).numpy()
+    rc, got = conv(x, w, N)
+    assert rc == F.Success
+    assert rel(got, oracle.corr2d_valid(x, w)) < TOL_CONV
