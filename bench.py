@@ -301,7 +301,28 @@ def conv_extras(F, synth, torch, dev, extra):
         "frac": round(260.5e6 / t / 1e9 / HBM_PEAK_GBS, 4), "algorithmic_bytes": 260500000,
         "traffic": profile_figure("conv_pipeline_configs4.md", "traffic_bytes_per_iteration"),
         "workload": "configs[4]: 16x32x256x256 * 32x32x9x9 -> 16x32x248x248, 32-point windows"}
-    del ws4
+    # the layer's other two passes on the same tiled image
+    gi4, gw4 = torch.empty_like(x4), torch.empty_like(w4)
+    vgi4, vgw4 = F.view(gi4), F.view(gw4)
+    wsb = torch.empty(max(F.conv_workspace_image(1, 16, 32, 32, 256, 256, 9, 9, 32),
+                          F.conv_workspace_image(2, 16, 32, 32, 256, 256, 9, 9, 32)),
+                      dtype=torch.uint8, device=dev)
+
+    def layer4_bprop():
+        if L.fbfft_conv_bprop(ctypes.byref(v4[2]), ctypes.byref(v4[1]), ctypes.byref(vgi4), 32,
+                              ctypes.c_void_p(wsb.data_ptr()), wsb.numel(), stream) != 0:
+            raise RuntimeError("fbfft_conv_bprop (tiled) failed")
+
+    def layer4_accgrad():
+        if L.fbfft_conv_accgrad(ctypes.byref(v4[0]), ctypes.byref(v4[2]), ctypes.byref(vgw4), 32,
+                                ctypes.c_float(1.0), 0, ctypes.c_void_p(wsb.data_ptr()), wsb.numel(),
+                                stream) != 0:
+            raise RuntimeError("fbfft_conv_accgrad (tiled) failed")
+    _, t = timed(layer4_bprop, 40, 20, torch)
+    extra["conv_layer_configs4_bprop_ms_per_iter"] = round(t * 1e3, 4)
+    _, t = timed(layer4_accgrad, 40, 20, torch)
+    extra["conv_layer_configs4_accgrad_ms_per_iter"] = round(t * 1e3, 4)
+    del ws4, wsb, gi4, gw4
     # the other two passes (o4 as gradOutput): accGradParameters on the same descriptors,
     # updateGradInput on its own grid of disjoint gradInput windows
     bins, bouts, nbp = F.make_tile_grid(x4, o4, 9, 9, 32, F.FFT_UpdateGradInput)
