@@ -37,6 +37,19 @@ inline int launchStatus() {
   return hipGetLastError() == hipSuccess ? FBFFT_SUCCESS : FBFFT_HIP_ERROR;
 }
 
+// compute units of the current device (256 on MI355X); queried once
+inline int computeUnits() {
+  static const int n = [] {
+    int dev = 0, cus = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
+        cus <= 0)
+      cus = 256;
+    return cus;
+  }();
+  return n;
+}
+
 // kernel launchers implemented in the .hip files (return an fbfft_error)
 int launchFft2dSmallForward(int N, const RealView& real, const CplxView& cplx, int padL, int padU,
                             hipStream_t s, bool packed = false);

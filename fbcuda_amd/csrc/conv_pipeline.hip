@@ -80,6 +80,16 @@ struct PlaneSet {
   int padU0, padL0;
 };
 
+// Orders the LDS accesses of one wave: what its lanes wrote before is what its lanes
+// read after.  The lanes that share a plane sit in one wave, and a wave's LDS
+// instructions execute in order, so the passes over a plane need no workgroup barrier
+// between them - only the compiler has to keep the accesses in program order.
+__device__ __forceinline__ void planeSync() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
 struct PlaneWindow {
   float* p;
   int h, w, padL, padU;
@@ -155,7 +165,7 @@ __device__ __forceinline__ void forwardBinMajorBody(const ForwardJob& job, int w
   }
   c32* plane = lds + s * PSZ;
   columnPassForward<N>(z0, z1, plane, l);
-  __syncthreads();
+  planeSync();  // the lanes of a plane sit in one wave
   rowPassInPlace<N, true>(plane, l);
   __syncthreads();
 
@@ -191,64 +201,88 @@ __device__ __forceinline__ void forwardBinMajorBody(const ForwardJob& job, int w
 }
 
 // ---- 3. C[bin][i][j] -> planes (i, j), cropped ----
-template <int N, bool ACC>
+// A workgroup takes GROUPS (1 or 2) runs of SLOTS consecutive j of one i.  With two, the
+// second run's spectra are requested as soon as the first run's have been parked in
+// LDS, and fly under the first run's transforms and stores.
+template <int N, bool ACC, int GROUPS>
 __global__ __launch_bounds__(kT) void inverseBinMajor(const float2* Cs, int I, int Jp, PlaneSet out,
                                                       float scale) {
   using C = BMCfg<N>;
   constexpr int H = C::H, T = C::T, SLOTS = C::SLOTS, RS = C::RS, PSZ = C::PSZ;
+  constexpr int PER = C::BINS / T;
+  static_assert(C::BINS % T == 0, "bins divide evenly over the lane groups");
   __shared__ __align__(16) c32 lds[SLOTS * PSZ];
   const int t = threadIdx.x;
   const int s = t / T, l = t % T;
-  const int j0 = blockIdx.x * SLOTS;
   const int i = blockIdx.y;
-
   const int sp = t % SLOTS, bq = t / SLOTS;
-  {
-    // gather: every load is issued before the first LDS store
-    constexpr int PER = C::BINS / T;
-    static_assert(C::BINS % T == 0, "bins divide evenly over the lane groups");
-    c32* dstp = lds + sp * PSZ;
+  const long binStride = (long)I * Jp;
+  c32* plane = lds + s * PSZ;
+
+  // gather: every load of a run is issued before its first LDS store
+  auto request = [&](int j0, c32 (&in)[PER]) __attribute__((always_inline)) {
     const float2* src = Cs + (long)i * Jp + j0 + sp;
-    const long binStride = (long)I * Jp;
-    c32 in[PER];
     staticFor<PER>([&](auto uu) {
       constexpr int u = decltype(uu)::value;
       in[u] = src[(bq + T * u) * binStride];
     });
+  };
+  auto park = [&](const c32 (&in)[PER]) __attribute__((always_inline)) {
+    c32* dstp = lds + sp * PSZ;
     staticFor<PER>([&](auto uu) {
       constexpr int u = decltype(uu)::value;  // bin = bq + T*u: row u/2, column bq + T*(u%2)
       dstp[(u / 2) * RS + T * (u % 2) + bq] = in[u];
     });
-  }
-  __syncthreads();
-  c32* plane = lds + s * PSZ;
-  {  // virtual bins of row 0 back to the packed row: Q[x] = C0[x] + i CH[x],
-     // Q[N-x] = conj(C0[x]) + i conj(CH[x]); lane 0 sorts the four real values into
-     // Q[0] = (C0[0], CH[0]) and Q[N/2] = (C0[N/2], CH[N/2]).  The T lanes of a plane
-     // sit in one wave: all of them have read before any of them writes.
-    const c32 c0 = plane[l], cH = plane[T + l];
-    c32 q = c32{c0.x - cH.y, c0.y + cH.x}, qm = c32{c0.x + cH.y, cH.x - c0.y};
-    if (l == 0) {
-      q = c32{c0.x, cH.x};
-      qm = c32{c0.y, cH.y};
+  };
+  auto transformAndStore = [&](int j0) __attribute__((always_inline)) {
+    {  // virtual bins of row 0 back to the packed row: Q[x] = C0[x] + i CH[x],
+       // Q[N-x] = conj(C0[x]) + i conj(CH[x]); lane 0 sorts the four real values into
+       // Q[0] = (C0[0], CH[0]) and Q[N/2] = (C0[N/2], CH[N/2]).  The T lanes of a plane
+       // sit in one wave: all of them have read before any of them writes.
+      const c32 c0 = plane[l], cH = plane[T + l];
+      c32 q = c32{c0.x - cH.y, c0.y + cH.x}, qm = c32{c0.x + cH.y, cH.x - c0.y};
+      if (l == 0) {
+        q = c32{c0.x, cH.x};
+        qm = c32{c0.y, cH.y};
+      }
+      plane[l] = q;
+      plane[l == 0 ? H : N - l] = qm;
     }
-    plane[l] = q;
-    plane[l == 0 ? H : N - l] = qm;
-  }
+    planeSync();
+    rowPassInPlace<N, false>(plane, l);
+    planeSync();
+    c32 z0[H], z1[H];
+    columnPassInverse<N>(plane, l, z0, z1);
+    const int j = j0 + s;
+    // (Parking the cropped planes in LDS and writing them out as 16-byte runs - one
+    // contiguous stream for dense outputs, row quads for windows of a tiled image - was
+    // measured and is slower, 35.9 -> 36.6 us at configs[3] and 112 -> 131 us at
+    // configs[4]: the kernel waits on its own chain of phases, not on store requests.)
+    if (j < out.K) {  // out.K: number of valid output planes along j
+      const PlaneWindow win = planeWindow(out, i, j);
+      storeColumnsWindow<N, ACC>(win.p, out.sy, out.sx, win.h, win.w, win.padL, win.padU, l, z0,
+                                 z1, scale);
+    }
+  };
+
+  const int ja = blockIdx.x * GROUPS * SLOTS;
+  c32 in[PER];
+  request(ja, in);
+  park(in);
   __syncthreads();
-  rowPassInPlace<N, false>(plane, l);
-  __syncthreads();
-  c32 z0[H], z1[H];
-  columnPassInverse<N>(plane, l, z0, z1);
-  const int j = j0 + s;
-  // (Parking the cropped planes in LDS and writing them out as 16-byte runs - one
-  // contiguous stream for dense outputs, row quads for windows of a tiled image - was
-  // measured and is slower, 35.9 -> 36.6 us at configs[3] and 112 -> 131 us at
-  // configs[4]: the kernel waits on its own chain of phases, not on store requests.)
-  if (j < out.K) {  // out.K: number of valid output planes along j
-    const PlaneWindow win = planeWindow(out, i, j);
-    storeColumnsWindow<N, ACC>(win.p, out.sy, out.sx, win.h, win.w, win.padL, win.padU, l, z0, z1,
-                               scale);
+  if constexpr (GROUPS == 2) {
+    const int jb = ja + SLOTS;
+    const bool second = jb < Jp;  // the same for the whole workgroup
+    if (second) request(jb, in);
+    transformAndStore(ja);
+    if (second) {
+      __syncthreads();  // every wave has read the first run out of the plane buffers
+      park(in);
+      __syncthreads();
+      transformAndStore(jb);
+    }
+  } else {
+    transformAndStore(ja);
   }
 }
 
@@ -596,10 +630,21 @@ int runPipeline(PlaneSet x, PlaneSet y, PlaneSet out, bool conjY, float scale, b
     g.IT = ceilDiv(I, GI);
     binGemmDirect<GI><<<dim3(roundUp(bins * g.IT * g.JT, 8)), dim3(kT), 0, s>>>(g);
   }
-  if (accumulate)
-    inverseBinMajor<N, true><<<dim3(Jp / SL, I), dim3(kT), 0, s>>>(SC, I, Jp, out, scale);
-  else
-    inverseBinMajor<N, false><<<dim3(Jp / SL, I), dim3(kT), 0, s>>>(SC, I, Jp, out, scale);
+  // Two runs per workgroup pay when the paired launch still fills the chip for three
+  // rounds or more (two workgroups are resident per CU): 112 -> 108 us at configs[4],
+  // 1936 paired workgroups; at configs[3] pairing would leave 768 workgroups, one and a
+  // half rounds, and costs 35.5 -> 37.1 us.
+  if (Jp / SL >= 2 && (long)ceilDiv(Jp / SL, 2) * I >= 3L * 2 * computeUnits()) {
+    const dim3 igrid(ceilDiv(Jp / SL, 2), I);
+    if (accumulate)
+      inverseBinMajor<N, true, 2><<<igrid, dim3(kT), 0, s>>>(SC, I, Jp, out, scale);
+    else
+      inverseBinMajor<N, false, 2><<<igrid, dim3(kT), 0, s>>>(SC, I, Jp, out, scale);
+  } else if (accumulate) {
+    inverseBinMajor<N, true, 1><<<dim3(Jp / SL, I), dim3(kT), 0, s>>>(SC, I, Jp, out, scale);
+  } else {
+    inverseBinMajor<N, false, 1><<<dim3(Jp / SL, I), dim3(kT), 0, s>>>(SC, I, Jp, out, scale);
+  }
   return launchStatus();
 }
 

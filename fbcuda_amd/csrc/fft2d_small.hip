@@ -315,18 +315,6 @@ __global__ __launch_bounds__(64) void fft2dSmallInverse(CplxView cplx, RealView 
 // exposed, and folding it into the first round's waves (with their loads already
 // in flight) hides it.  Measured on 32 x 32 R2C: 26.9 -> 24.6 us at 16384 planes,
 // but 102 -> 113 us at 65536 planes, where other waves already cover the latency.
-int computeUnits() {
-  static const int n = [] {
-    int dev = 0, cus = 0;
-    if (hipGetDevice(&dev) != hipSuccess ||
-        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
-        cus <= 0)
-      cus = 256;
-    return cus;
-  }();
-  return n;
-}
-
 // (Measured across the switch, 32 x 32 R2C, us per launch paired / unpaired: 9216 planes
 // 16.6 / 16.0, 10240 17.0 / 17.4, 12288 17.8 / 19.5, 14336 19.1 / 22.0, 16384 22.7 / 24.1;
 // a variant that keeps one full round of waves and gives only some of them a second
