@@ -27,7 +27,7 @@ __host__ __device__ __forceinline__ bool inWindow(int y, int x, int padU, int pa
   return (unsigned)(y - padU) < (unsigned)h && (unsigned)(x - padL) < (unsigned)w;
 }
 
-inline int ceilDiv(int a, int b) { return (a + b - 1) / b; }
+__host__ __device__ inline int ceilDiv(int a, int b) { return (a + b - 1) / b; }
 
 inline bool aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
 
