@@ -7,26 +7,30 @@
 // Operands keep the reference layout: complex, xy innermost and contiguous, so
 // xy is the batch index of 'XY' independent small GEMMs and a coalesced global
 // access is a run of consecutive bins of one (row, col) element.  Accumulators
-// are needed for every bin of a run at once, which bounds the tile: a workgroup
-// of 8 waves owns a 64 x 64 tile of C for 8 consecutive bins (64-byte runs; the
-// other half of each line goes to the neighbouring workgroup on the same XCD),
-// wave w owning bin w: 4 MFMA 32x32 sub-tiles x 3 partial products = 192
-// accumulator registers per lane.
+// are needed for every bin of a run at once, which bounds the tile; a work item is
+// a tile of C for 8 consecutive bins (64-byte runs; the other half of each line goes
+// to the neighbouring workgroup on the same XCD).  Every path issues
+// v_mfma_f32_32x32x2_f32, three real products per complex product
+// (k1 = (Ar+Ai) Br, k2 = Ar (Bi-Br), k3 = Ai (Br+Bi); Cre = k1 - k3,
+// Cim = k1 + k2), holds 192 accumulator registers per lane and sends C through LDS
+// so that stores cover whole runs.  Only this contraction uses MFMA; it is the one
+// dense product of the convolution path.
 //
-// Per 4-deep slice of k the workgroup stages opA and opB in LDS split into real
-// and imaginary planes [bin][k][row] (conjugation folded into the sign of the
-// imaginary plane), two buffers deep, while the slice after next is in flight in
-// registers; each
-// wave then issues v_mfma_f32_32x32x2_f32, three real products per complex
-// product (k1 = (Ar+Ai) Br, k2 = Ar (Bi-Br), k3 = Ai (Br+Bi); Cre = k1 - k3,
-// Cim = k1 + k2).  C leaves through LDS
-// so that stores cover whole runs.  Only this contraction uses MFMA; it is the
-// one dense product of the convolution path.
+// Two kernels:
+//  * the fast path (transposeMMDirectKernel, further down) for operands whose runs of
+//    bin pairs are 16-byte aligned: 64 x 32 tiles, four waves of one bin pair each,
+//    slices of k copied from HBM into LDS without passing through registers, two
+//    workgroups per CU;
+//  * the register path (transposeMMKernel) for everything else and for packed row 0:
+//    a workgroup of 8 waves owns a 64 x 64 tile, wave w owning bin w.  Per 4-deep
+//    slice of k it parks opA and opB in LDS split into real and imaginary planes
+//    [bin][k][row] (conjugation folded into the sign of the imaginary plane, edges
+//    zeroed), two buffers deep, while the slice after next is in flight in registers.
 //
 // Packed spectra (fbfft_transpose_mm_packed): operands [..][..][N/2][N] whose row 0
 // holds P[x] = F0[x] + i FH[x], the spectra of the two real rows 0 and N/2 of an
 // N x N transform (the Unpack = false format of fbfft/FFT2D32.cuh:421-427).  Rows
-// 1 .. N/2-1 are plain bins and go through the kernel above.  Row 0 follows the
+// 1 .. N/2-1 are plain bins and go through the register path.  Row 0 follows the
 // product rule of fbfft/FFTIteratedConvolution.cuh:161-186: unpack both operands,
 // multiply F0 with F0 and FH with FH, re-pack.  The PACKED0 variant of the kernel
 // does that on the way into and out of LDS: a workgroup takes four x (0 < x < N/2)
@@ -34,7 +38,6 @@
 // P[N-x] when a slice is parked; the epilogue combines C0[x] and CH[x] into P[x] and
 // P[N-x].  x = 0 pairs with x = N/2: both hold two real values, which multiply
 // component by component (no cross terms).
-#include <cstdlib>
 #include <utility>
 
 #include "common.h"
@@ -51,11 +54,7 @@ constexpr int CSTR = XB + 1;  // padded bin stride of the C staging buffer (comp
 // Shape of a work item.  WAVES waves share a TI x TJ tile of C for 8 consecutive
 // bins; wave w owns bins w, w + WAVES, ...: (TI/32) x (TJ/32) MFMA sub-tiles x 3
 // partial products x 16 registers for each of its bins - 192 accumulator registers
-// in both shapes below.
-//   Wide (64 x 64, 8 waves of one bin): fewest operand re-reads; its 512 lanes fill a
-//     CU, so a CU either multiplies or writes C out.
-//   Half (64 x 32, 4 waves of two bins): two workgroups share a CU and one's C leaves
-//     while the other multiplies.
+// for Wide (64 x 64, 8 waves of one bin), whose 512 lanes fill a CU.
 template <int TI_, int TJ_, int WAVES_>
 struct Geo {
   static constexpr int TI = TI_, TJ = TJ_, WAVES = WAVES_, THREADS = 64 * WAVES_;
@@ -73,7 +72,6 @@ struct Geo {
   static_assert(CR % 8 == 0 && 32 % CR == 0 && XB % WAVES == 0, "shape");
 };
 using Wide = Geo<64, 64, 8>;
-using Half = Geo<64, 32, 4>;
 
 struct MMArgs {
   const float* A;
@@ -426,8 +424,7 @@ __device__ __forceinline__ int logicalWorkItem(int total) {
   return (blockIdx.x % 8) * per + blockIdx.x / 8;
 }
 
-// Both shapes are built for two waves per SIMD (256 registers a lane): one Wide
-// workgroup or two Half workgroups per CU.
+// Built for two waves per SIMD (256 registers a lane): one Wide workgroup per CU.
 template <typename G, bool VEC4>
 __global__ __launch_bounds__(G::THREADS) __attribute__((amdgpu_waves_per_eu(2, 2))) void transposeMMKernel(MMArgs a, int total) {
   __shared__ __align__(8) float lds[G::LDS_FLOATS];  // two slice buffers; later the C staging area
@@ -459,7 +456,7 @@ __global__ __launch_bounds__(G::THREADS) __attribute__((amdgpu_waves_per_eu(2, 2
 
 // ---- fast path: operands and C 16-byte aligned in every run of bin pairs, XY even ----
 //
-// Half-shape work items whose slices go from HBM straight into LDS (global_load_lds,
+// Half-size work items (64 x 32) whose slices go from HBM straight into LDS (global_load_lds,
 // 16 bytes per lane): no staging registers, no parking instructions - the side work
 // per slice shrinks from some hundred vector instructions to six loads and their
 // addresses, and vector instructions do not hide under the matrix pipeline here (the
@@ -576,6 +573,9 @@ __device__ __forceinline__ void transposeMMDirectBody(const MMArgs& a, int logic
       __syncthreads();
     }
     issue(refillA, refillB, sl + 2);
+    // left alone the compiler sinks the requests to the end of the step, which halves
+    // the time they have to arrive
+    __builtin_amdgcn_sched_barrier(0);
     const float4* flatA = &curA.v[0][0][0];
     const float4* flatB = &curB.v[0][0][0];
     float4 av[KC / 2][2], bv[KC / 2];
@@ -725,12 +725,6 @@ bool storesAsFloat4(const float* C, long c0, long c1) {
 }
 
 
-// Half-size work items once they outnumber the slots of two workgroups per CU
-bool halfItems(const MMArgs& m) {
-  if (const char* e = getenv("FBFFT_EXP_MM")) return atoi(e) == 2;
-  return false;
-}
-
 template <typename G>
 int launchPlain(const MMArgs& m, bool vec4, hipStream_t s) {
   const int total = workItems<G>(m);
@@ -764,13 +758,12 @@ int launchTransposeMM(const float* A, long a0, long a1, const float* B, long b0,
   const MMArgs m = makeArgs(A, a0, a1, B, b0, b1, C, c0, c1, I, J, K, XY, conjA, conjB, accumulate,
                             invNorm, ceilDiv(XY, XB));
   const bool vec4 = movesAsFloat4(A, a0, a1, B, b0, b1, XY);
-  const int mode = getenv("FBFFT_EXP_MM") ? atoi(getenv("FBFFT_EXP_MM")) : 3;
-  if (mode == 3 && vec4 && storesAsFloat4(C, c0, c1)) {
+  if (vec4 && storesAsFloat4(C, c0, c1)) {
     const int total = directWorkItems(m);
     transposeMMDirectKernel<<<dim3((total + 7) / 8 * 8), dim3(DTHREADS), 0, s>>>(m, total);
     return launchStatus();
   }
-  return halfItems(m) ? launchPlain<Half>(m, vec4, s) : launchPlain<Wide>(m, vec4, s);
+  return launchPlain<Wide>(m, vec4, s);
 }
 
 // The same contraction on packed spectra [d0][d1][N/2][N][2]: rows 1 .. N/2-1 as
@@ -786,8 +779,7 @@ int launchTransposeMMPacked(const float* A, long a0, long a1, const float* B, lo
   const MMArgs row0 = makeArgs(A, a0, a1, B, b0, b1, C, c0, c1, I, J, K, N, conjA, conjB,
                                accumulate, invNorm, N / XB);
   const bool vec4 = movesAsFloat4(A + 2 * N, a0, a1, B + 2 * N, b0, b1, XY);
-  return halfItems(mainRows) ? launchPacked<Half>(mainRows, row0, vec4, s)
-                             : launchPacked<Wide>(mainRows, row0, vec4, s);
+  return launchPacked<Wide>(mainRows, row0, vec4, s);
 }
 
 }  // namespace fbfft_amd

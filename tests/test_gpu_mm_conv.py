@@ -374,3 +374,27 @@ def test_conv_fprop_many_full_tiles(oracle, Cin):
     rc, got = conv(x, w, N)
     assert rc == F.Success
     assert rel(got, oracle.corr2d_valid(x, w)) < TOL_CONV
+
+
+@pytest.mark.parametrize("conjA,conjB", ROLES)
+@pytest.mark.parametrize("K", [1, 2, 3, 4, 6, 7, 13])
+@pytest.mark.parametrize("shape", [(1, 2), (1, 8), (5, 2), (3, 8), (2, 17)])
+def test_mm_aligned_operands_k_tails(oracle, conjA, conjB, K, shape):
+    """Even bin counts in contiguous tensors take the kernel that copies slices of four
+    k straight into LDS: every remainder of K modulo four, bin counts below, at and
+    between multiples of the eight bins of a work item, tiles with clamped rows."""
+    I, J = 70, 37
+    xy = shape[0] * shape[1]
+    A = synth.normal(((K, I) if conjA else (I, K)) + shape + (2,), seed=11 + K).numpy()
+    B = synth.normal(((J, K) if conjB else (K, J)) + shape + (2,), seed=12 + K).numpy()
+    C0 = synth.normal((I, J) + shape + (2,), seed=13).numpy()
+    A3 = A.reshape(A.shape[0], A.shape[1], xy, 2)
+    B3 = B.reshape(B.shape[0], B.shape[1], xy, 2)
+    for start in (None, C0):
+        rc, got = mm(A, B, conjA, conjB, 0.25, C0=start)
+        assert rc == F.Success
+        want = oracle.transpose_mm(A3, B3, conjA, conjB, 0.25,
+                                   C=None if start is None else start.reshape(I, J, xy, 2))
+        assert rel(got.reshape(I, J, xy, 2), want) < TOL_FFT
+        if start is None:
+            assert rel(got.reshape(I, J, xy, 2), oracle.transpose_mm64(A3, B3, conjA, conjB, 0.25)) < TOL_FFT
