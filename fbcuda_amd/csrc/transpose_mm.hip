@@ -470,11 +470,13 @@ __global__ __launch_bounds__(G::THREADS) __attribute__((amdgpu_waves_per_eu(2, 2
 // pair c ^ (r / 4) of row r: four neighbouring lanes read one 64-byte run, and the 16
 // rows of one pair land in 16 different 16-byte bank groups, so the 16-byte operand
 // reads (32 rows of one pair at two k) meet no bank conflicts.
-constexpr int DTI = 64, DTJ = 32, DTHREADS = 256;
-constexpr int DLOADS = DTI / 16 + DTJ / 16;  // global->LDS instructions per wave and slice
-constexpr int DCR = 8;                       // rows of C per staging chunk
+constexpr int DTJ = 32, DTHREADS = 256;
+// rows of C per staging chunk: 8, or 4 where the stages (which the staging areas
+// share their memory with) are small
+constexpr int directChunkRows(int DTI) { return DTI == 64 ? 8 : 4; }
 
 // [k][group of 16 rows][slot]; A and B of a stage are separate LDS variables
+template <int DTI>
 struct DirectA {
   float4 v[KC][DTI / 16][64];
 };
@@ -482,9 +484,10 @@ struct DirectB {
   float4 v[KC][DTJ / 16][64];
 };
 // stages 0 and 1 of A double as the staging areas of C
+template <int DTI>
 struct DirectA0 {
   float4 v[KC][DTI / 16][64];
-  float4 pad[(DCR * DTJ * CSTR * sizeof(float2) - sizeof(DirectA)) / sizeof(float4)];
+  float4 pad[(directChunkRows(DTI) * DTJ * CSTR * sizeof(float2) - sizeof(DirectA<DTI>)) / sizeof(float4)];
 };
 
 __device__ __forceinline__ int directSlot(int row16, int pair) { return 4 * row16 + (pair ^ (row16 / 4)); }
@@ -494,13 +497,18 @@ __device__ __forceinline__ void loadToLds(const float* src, float4* ldsWaveBase)
                                    (__attribute__((address_space(3))) void*)ldsWaveBase, 16, 0, 0);
 }
 
+// DTI: rows of the tile, 64, or 32 (one sub-tile per bin: 96 accumulator registers,
+// three workgroups per CU, C staged in chunks of four rows)
+template <int DTI>
 __device__ __forceinline__ void transposeMMDirectBody(const MMArgs& a, int logical) {
+  constexpr int SI = DTI / 32, DCR = directChunkRows(DTI);
+  constexpr int DLOADS = DTI / 16 + DTJ / 16;  // global->LDS instructions per wave and slice
   // Six separate variables, not arrays of stages: the compiler tracks pending
   // global->LDS loads per LDS variable (and only for accesses that start at a
   // variable's first byte plus a run-time offset), so reading one stage does not wait
   // for the loads still in flight into the other two.
-  __shared__ __align__(16) DirectA0 stageA0, stageA1;
-  __shared__ __align__(16) DirectA stageA2;
+  __shared__ __align__(16) DirectA0<DTI> stageA0, stageA1;
+  __shared__ __align__(16) DirectA<DTI> stageA2;
   __shared__ __align__(16) DirectB stageB0, stageB1, stageB2;
   const int t = threadIdx.x;
   const int lane = t % 64, w = __builtin_amdgcn_readfirstlane(t / 64);
@@ -542,11 +550,11 @@ __device__ __forceinline__ void transposeMMDirectBody(const MMArgs& a, int logic
 
   // [bin of the pair][sub-tile of A]; a b = (k1 - k3) + i (k1 + k2) for
   //   k1 = (ar + sA ai) br,  k2 = ar (sB bi - br),  k3 = ai (sA br + sA sB bi)
-  floatx16 k1[2][2], k2[2][2], k3[2][2];
+  floatx16 k1[2][SI], k2[2][SI], k3[2][SI];
 #pragma unroll
   for (int h = 0; h < 2; ++h)
 #pragma unroll
-    for (int si = 0; si < 2; ++si)
+    for (int si = 0; si < SI; ++si)
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         k1[h][si][r] = 0.f;
@@ -567,7 +575,7 @@ __device__ __forceinline__ void transposeMMDirectBody(const MMArgs& a, int logic
     if ((sl + 1) * KC > a.K) {
       // last, partial slice: the k beyond K hold copies of k = K-1
       for (int kz = a.K - sl * KC; kz < KC; ++kz) {
-        curA.v[kz][t / 64][t % 64] = float4{0.f, 0.f, 0.f, 0.f};
+        if (t < 64 * (DTI / 16)) curA.v[kz][t / 64][t % 64] = float4{0.f, 0.f, 0.f, 0.f};
         if (t < 64 * (DTJ / 16)) curB.v[kz][t / 64][t % 64] = float4{0.f, 0.f, 0.f, 0.f};
       }
       __syncthreads();
@@ -578,13 +586,14 @@ __device__ __forceinline__ void transposeMMDirectBody(const MMArgs& a, int logic
     __builtin_amdgcn_sched_barrier(0);
     const float4* flatA = &curA.v[0][0][0];
     const float4* flatB = &curB.v[0][0][0];
-    float4 av[KC / 2][2], bv[KC / 2];
+    float4 av[KC / 2][SI], bv[KC / 2];
 #pragma unroll
     for (int s2 = 0; s2 < KC / 2; ++s2) {
       // one flat index per read: address chains of several steps lose the mark that
       // ties an access to its LDS variable
-      av[s2][0] = flatA[readA + (2 * s2) * (DTI / 16) * 64];
-      av[s2][1] = flatA[readA + (2 * s2) * (DTI / 16) * 64 + 2 * 64];
+#pragma unroll
+      for (int si = 0; si < SI; ++si)
+        av[s2][si] = flatA[readA + (2 * s2) * (DTI / 16) * 64 + 2 * si * 64];
       bv[s2] = flatB[readB + (2 * s2) * (DTJ / 16) * 64];
     }
 #pragma unroll
@@ -595,7 +604,7 @@ __device__ __forceinline__ void transposeMMDirectBody(const MMArgs& a, int logic
         const float bd = __builtin_fmaf(sB, bi[h], -br[h]);
         const float bs = sA * __builtin_fmaf(sB, bi[h], br[h]);
 #pragma unroll
-        for (int si = 0; si < 2; ++si) {
+        for (int si = 0; si < SI; ++si) {
           const float ar = h ? av[s2][si].z : av[s2][si].x, ai = h ? av[s2][si].w : av[s2][si].y;
           const float as = __builtin_fmaf(sA, ai, ar);
           k1[h][si] = __builtin_amdgcn_mfma_f32_32x32x2f32(as, br[h], k1[h][si], 0, 0, 0);
@@ -630,27 +639,33 @@ __device__ __forceinline__ void transposeMMDirectBody(const MMArgs& a, int logic
   // parked while this one is stored.
   float2* stg[2] = {reinterpret_cast<float2*>(&stageA0), reinterpret_cast<float2*>(&stageA1)};
   const int col = lane % 32, hh = lane / 32;
+  // chunk n: rows 32 si + 8 c + 4 half .. of the tile; with four rows per chunk only
+  // the lanes of one half hold them
+  constexpr int CHUNKS = 32 / DCR * SI, PER8 = 8 / DCR;
   auto park = [&](auto nn) __attribute__((always_inline)) {
-    constexpr int n = decltype(nn)::value, si = n / 4, c = n % 4;
-    float2* st = stg[n % 2];  // [8 rows][32 cols][CSTR] complex
+    constexpr int n = decltype(nn)::value, si = n / (4 * PER8), c = n / PER8 % 4, half = n % PER8;
+    float2* st = stg[n % 2];  // [DCR rows][32 cols][CSTR] complex
+    if (DCR == 8 || hh == half) {
 #pragma unroll
-    for (int h = 0; h < 2; ++h)
+      for (int h = 0; h < 2; ++h)
 #pragma unroll
-      for (int rr = 0; rr < 4; ++rr) {
-        const float v1 = k1[h][si][4 * c + rr], v2 = k2[h][si][4 * c + rr],
-                    v3 = k3[h][si][4 * c + rr];
-        st[((4 * hh + rr) * DTJ + col) * CSTR + 2 * w + h] = float2{v1 - v3, v1 + v2};
-      }
+        for (int rr = 0; rr < 4; ++rr) {
+          const float v1 = k1[h][si][4 * c + rr], v2 = k2[h][si][4 * c + rr],
+                      v3 = k3[h][si][4 * c + rr];
+          st[(((DCR == 8 ? 4 * hh : 0) + rr) * DTJ + col) * CSTR + 2 * w + h] =
+              float2{v1 - v3, v1 + v2};
+        }
+    }
   };
   const int q = t % 4;
   auto store = [&](auto nn) __attribute__((always_inline)) {
-    constexpr int n = decltype(nn)::value, si = n / 4, c = n % 4;
+    constexpr int n = decltype(nn)::value, si = n / (4 * PER8), c = n / PER8 % 4, half = n % PER8;
     const float2* st = stg[n % 2];
 #pragma unroll
     for (int pass = 0; pass < DCR * DTJ * 4 / DTHREADS; ++pass) {
       const int e = t / 4 + (DTHREADS / 4) * pass;
       const int row = e / DTJ, cc = e % DTJ;
-      const int i = i0 + 32 * si + DCR * c + row, j = j0 + cc, x = x0 + 2 * q;
+      const int i = i0 + 32 * si + 8 * c + 4 * half + row, j = j0 + cc, x = x0 + 2 * q;
       const float2 c0 = st[e * CSTR + 2 * q], c1 = st[e * CSTR + 2 * q + 1];
       float4 acc{c0.x, c0.y, c1.x, c1.y};
       if (i < a.I && j < a.J && x < a.XY) {
@@ -670,23 +685,26 @@ __device__ __forceinline__ void transposeMMDirectBody(const MMArgs& a, int logic
   __syncthreads();  // the last slice is consumed by everybody
   park(std::integral_constant<int, 0>{});
   __syncthreads();
-  unrolled<8>([&](auto nn) {
+  unrolled<CHUNKS>([&](auto nn) {
     constexpr int n = decltype(nn)::value;
-    if constexpr (n + 1 < 8) park(std::integral_constant<int, n + 1>{});
+    if constexpr (n + 1 < CHUNKS) park(std::integral_constant<int, n + 1>{});
     store(nn);
-    if constexpr (n + 1 < 8) __syncthreads();
+    if constexpr (n + 1 < CHUNKS) __syncthreads();
   });
 }
 
+template <int DTI>
 inline int directWorkItems(const MMArgs& a) {
   return a.chunks * ceilDiv(a.J, DTJ) * ceilDiv(a.I, DTI);
 }
 
-// two workgroups per CU: one's C leaves while the other multiplies
-__global__ __launch_bounds__(DTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2))) void transposeMMDirectKernel(
-    MMArgs a, int total) {
+// two (64 rows) or three (32 rows) workgroups per CU: one's C leaves while the others
+// multiply
+template <int DTI>
+__global__ __launch_bounds__(DTHREADS) __attribute__((amdgpu_waves_per_eu(DTI == 64 ? 2 : 3, DTI == 64 ? 2 : 3)))
+void transposeMMDirectKernel(MMArgs a, int total) {
   const int logical = logicalWorkItem(total);
-  if (logical < total) transposeMMDirectBody(a, logical);
+  if (logical < total) transposeMMDirectBody<DTI>(a, logical);
 }
 
 MMArgs makeArgs(const float* A, long a0, long a1, const float* B, long b0, long b1, float* C,
@@ -759,8 +777,20 @@ int launchTransposeMM(const float* A, long a0, long a1, const float* B, long b0,
                             invNorm, ceilDiv(XY, XB));
   const bool vec4 = movesAsFloat4(A, a0, a1, B, b0, b1, XY);
   if (vec4 && storesAsFloat4(C, c0, c1)) {
-    const int total = directWorkItems(m);
-    transposeMMDirectKernel<<<dim3((total + 7) / 8 * 8), dim3(DTHREADS), 0, s>>>(m, total);
+    // Equal work items are dealt to the CUs in whole numbers: the launch lasts as
+    // long as the fullest CU.  32-row tiles re-read B twice as often and pay more per
+    // matrix instruction, so they are taken only where they even the load out
+    // (configs[3]: 816 items of 64 rows are 3.19 per CU, four on the fullest - 72 us;
+    // 1632 of 32 rows are 6.4, seven on the fullest - 68 us; at 2, 4 or 8 items of 64
+    // rows per CU the larger tile wins by 3-9 %).
+    const int cus = computeUnits();
+    auto evenness = [&](int items) { return (double)items / cus / ceilDiv(items, cus); };
+    const int items64 = directWorkItems<64>(m), items32 = directWorkItems<32>(m);
+    if (evenness(items32) > evenness(items64) + 0.05) {
+      transposeMMDirectKernel<32><<<dim3((items32 + 7) / 8 * 8), dim3(DTHREADS), 0, s>>>(m, items32);
+    } else {
+      transposeMMDirectKernel<64><<<dim3((items64 + 7) / 8 * 8), dim3(DTHREADS), 0, s>>>(m, items64);
+    }
     return launchStatus();
   }
   return launchPlain<Wide>(m, vec4, s);

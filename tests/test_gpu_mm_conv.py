@@ -398,3 +398,21 @@ def test_mm_aligned_operands_k_tails(oracle, conjA, conjB, K, shape):
         assert rel(got.reshape(I, J, xy, 2), want) < TOL_FFT
         if start is None:
             assert rel(got.reshape(I, J, xy, 2), oracle.transpose_mm64(A3, B3, conjA, conjB, 0.25)) < TOL_FFT
+
+
+@pytest.mark.parametrize("I,J,K,shape", [
+    (128, 128, 5, (16, 32)),   # 512 work items of 64 x 32: two per CU, the larger tile
+    (128, 96, 6, (17, 32)),    # 408 of them: uneven, the smaller tile
+])
+def test_mm_both_tile_shapes_of_the_aligned_path(oracle, I, J, K, shape):
+    """The aligned path picks 64- or 32-row tiles by how evenly the work items spread
+    over the CUs; one layer for each choice, both roles with a conjugation."""
+    xy = shape[0] * shape[1]
+    for conjA, conjB in ROLES[:2]:
+        A = synth.normal(((K, I) if conjA else (I, K)) + shape + (2,), seed=21).numpy()
+        B = synth.normal(((J, K) if conjB else (K, J)) + shape + (2,), seed=22).numpy()
+        rc, got = mm(A, B, conjA, conjB, 0.5)
+        assert rc == F.Success
+        want = oracle.transpose_mm(A.reshape(A.shape[0], A.shape[1], xy, 2),
+                                   B.reshape(B.shape[0], B.shape[1], xy, 2), conjA, conjB, 0.5)
+        assert rel(got.reshape(I, J, xy, 2), want) < TOL_FFT
