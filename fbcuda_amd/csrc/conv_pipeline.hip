@@ -47,13 +47,17 @@ namespace fbfft_amd {
 namespace {
 
 constexpr int kT = 256;
+#ifndef EXP_KTF
+#define EXP_KTF 256
+#endif
+constexpr int kTF = EXP_KTF;  // lanes of a transform workgroup
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
 template <int N>
 struct BMCfg {
   static constexpr int H = N / 2;
   static constexpr int T = N / 2;
-  static constexpr int SLOTS = kT / T;                 // planes per workgroup
+  static constexpr int SLOTS = kTF / T;                // planes per workgroup
   static constexpr int RS = PlaneCfg<N>::RS;
   // plane stride in LDS (complex): 16-byte aligned, and 4 banks mod 32 so that the
   // transposed accesses (16 or more planes at the same bin) spread over the banks
@@ -136,7 +140,7 @@ template <int N, int PAIRS, int GROUPS>
 __device__ __forceinline__ void forwardBinMajorBody(const ForwardJob& job, int wg, c32* lds);
 
 template <int N, int PAIRS_A, int PAIRS_B, int GROUPS>
-__global__ __launch_bounds__(kT) void forwardBinMajor(ForwardJob a, ForwardJob b) {
+__global__ __launch_bounds__(kTF) void forwardBinMajor(ForwardJob a, ForwardJob b) {
   __shared__ __align__(16) c32 lds[BMCfg<N>::SLOTS * BMCfg<N>::PSZ];
   const int nA = a.rowGroups * a.Kp;
   if ((int)blockIdx.x < nA)
@@ -233,8 +237,8 @@ __device__ __forceinline__ void forwardBinMajorBody(const ForwardJob& job, int w
 // A workgroup takes GROUPS (1 or 2) runs of SLOTS consecutive j of one i.  With two, the
 // second run's spectra are requested as soon as the first run's have been parked in
 // LDS, and fly under the first run's transforms and stores.
-template <int N, bool ACC, int GROUPS>
-__global__ __launch_bounds__(kT) void inverseBinMajor(const float2* Cs, int I, int Jp, PlaneSet out,
+template <int N, bool ACC, int GROUPS, bool PAIRS>
+__global__ __launch_bounds__(kTF) void inverseBinMajor(const float2* Cs, int I, int Jp, PlaneSet out,
                                                       float scale) {
   using C = BMCfg<N>;
   constexpr int H = C::H, T = C::T, SLOTS = C::SLOTS, RS = C::RS, PSZ = C::PSZ;
@@ -289,8 +293,8 @@ __global__ __launch_bounds__(kT) void inverseBinMajor(const float2* Cs, int I, i
     // configs[4]: the kernel waits on its own chain of phases, not on store requests.)
     if (j < out.K) {  // out.K: number of valid output planes along j
       const PlaneWindow win = planeWindow(out, i, j);
-      storeColumnsWindow<N, ACC>(win.p, out.sy, out.sx, win.h, win.w, win.padL, win.padU, l, z0,
-                                 z1, scale);
+      storeColumnsWindow<N, ACC, false, PAIRS>(win.p, out.sy, out.sx, win.h, win.w, win.padL,
+                                               win.padU, l, z0, z1, scale);
     }
   };
 
@@ -576,15 +580,21 @@ __global__ __launch_bounds__(kT, 4) void binGemmRegs(GemmArgs g) {
 
 inline int roundUp(int a, int b) { return (a + b - 1) / b * b; }
 
-// Which operand takes the 128-wide side of the GEMM tile: the assignment with
-// fewer padded tile elements.
-inline bool swapRoles(int I, int J) {
+// Which operand takes the 128-wide side of the GEMM tile (and with it the role of i, the
+// slow index of C[bin][i][j]).  Results cut into windows of a larger image (outTiled)
+// always put the window index on j: the inverse kernel transforms 16 consecutive j per
+// workgroup, and 16 neighbouring windows of one output plane store whole stretches of
+// image rows where 16 output planes of one window store 24-float pieces 248 floats apart
+// (configs[4]: 337 -> 308 us per forward pass).  Otherwise: the assignment with fewer
+// padded tile elements.
+inline bool swapRoles(int I, int J, bool outTiled) {
+  if (outTiled) return true;
   return (long)roundUp(J, GI) * roundUp(I, GJ2) < (long)roundUp(I, GI) * roundUp(J, GJ2);
 }
 
 template <int N>
-size_t workspaceFloat2(int I, int J, int K) {
-  if (swapRoles(I, J)) std::swap(I, J);
+size_t workspaceFloat2(int I, int J, int K, bool outTiled) {
+  if (swapRoles(I, J, outTiled)) std::swap(I, J);
   const int SL = BMCfg<N>::SLOTS, bins = BMCfg<N>::BINS;
   const int Ip = roundUp(I, SL), Jp = roundUp(J, SL), Kp = roundUp(K, 8);
   return (size_t)bins * ((size_t)Kp * Ip + (size_t)Kp * Jp + (size_t)I * Jp);
@@ -598,7 +608,7 @@ int runPipeline(PlaneSet x, PlaneSet y, PlaneSet out, bool conjY, float scale, b
   using C = BMCfg<N>;
   const int SL = C::SLOTS, bins = C::BINS;
   float xSign = 1.0f, ySign = conjY ? 1.0f : -1.0f;
-  if (swapRoles(x.R, y.R)) {
+  if (swapRoles(x.R, y.R, out.tiled != 0)) {
     // G[j][i] = sum_k op(Y[j]) * conj(conj X[i])
     std::swap(x, y);
     xSign = conjY ? -1.0f : 1.0f;
@@ -630,13 +640,13 @@ int runPipeline(PlaneSet x, PlaneSet y, PlaneSet out, bool conjY, float scale, b
   auto launchForward = [&](auto groups) {
     constexpr int G = decltype(groups)::value;
     if (pa && pb)
-      forwardBinMajor<N, 1, 1, G><<<fgrid, dim3(kT), 0, s>>>(ja, jb);
+      forwardBinMajor<N, 1, 1, G><<<fgrid, dim3(kTF), 0, s>>>(ja, jb);
     else if (pa)
-      forwardBinMajor<N, 1, 0, G><<<fgrid, dim3(kT), 0, s>>>(ja, jb);
+      forwardBinMajor<N, 1, 0, G><<<fgrid, dim3(kTF), 0, s>>>(ja, jb);
     else if (pb)
-      forwardBinMajor<N, 0, 1, G><<<fgrid, dim3(kT), 0, s>>>(ja, jb);
+      forwardBinMajor<N, 0, 1, G><<<fgrid, dim3(kTF), 0, s>>>(ja, jb);
     else
-      forwardBinMajor<N, 0, 0, G><<<fgrid, dim3(kT), 0, s>>>(ja, jb);
+      forwardBinMajor<N, 0, 0, G><<<fgrid, dim3(kTF), 0, s>>>(ja, jb);
   };
   if (two)
     launchForward(std::integral_constant<int, 2>{});
@@ -661,7 +671,7 @@ int runPipeline(PlaneSet x, PlaneSet y, PlaneSet out, bool conjY, float scale, b
   // Up to 32 columns the LDS kernels' 64-column tiles would be half empty; the register
   // kernel drops its idle sub-tiles (configs[4], 1936 x 32 x 32 per bin: 146 -> 139 us.
   // At configs[3], 128 x 192 x 64 per bin, it is the slower one: 64 against 58 us.)
-  if (Jp <= 32) {
+  if (Jp <= 32 || I <= 32) {
     g.IT = ceilDiv(I, 64);
     binGemmRegs<<<dim3(roundUp(bins * g.IT * g.JT, 8)), dim3(kT), 0, s>>>(g);
   } else if (small) {
@@ -675,17 +685,31 @@ int runPipeline(PlaneSet x, PlaneSet y, PlaneSet out, bool conjY, float scale, b
   // rounds or more (two workgroups are resident per CU): 112 -> 108 us at configs[4],
   // 1936 paired workgroups; at configs[3] pairing would leave 768 workgroups, one and a
   // half rounds, and costs 35.5 -> 37.1 us.
-  if (Jp / SL >= 2 && (long)ceilDiv(Jp / SL, 2) * I >= 3L * 2 * computeUnits()) {
-    const dim3 igrid(ceilDiv(Jp / SL, 2), I);
-    if (accumulate)
-      inverseBinMajor<N, true, 2><<<igrid, dim3(kT), 0, s>>>(SC, I, Jp, out, scale);
+  const bool pairedRuns = Jp / SL >= 2 && (long)ceilDiv(Jp / SL, 2) * I >= 3L * 2 * computeUnits();
+  const dim3 igrid(pairedRuns ? ceilDiv(Jp / SL, 2) : Jp / SL, I);
+  // windows whose rows start on 8-byte boundaries with an even width: a lane stores its
+  // two columns of a row as one 8-byte word
+  const bool po = movesAsPairs(out);
+  auto launchInverse = [&](auto acc, auto groups, auto pairs) {
+    inverseBinMajor<N, decltype(acc)::value, decltype(groups)::value, decltype(pairs)::value>
+        <<<igrid, dim3(kTF), 0, s>>>(SC, I, Jp, out, scale);
+  };
+  auto withPairs = [&](auto acc, auto groups) {
+    if (po)
+      launchInverse(acc, groups, std::true_type{});
     else
-      inverseBinMajor<N, false, 2><<<igrid, dim3(kT), 0, s>>>(SC, I, Jp, out, scale);
-  } else if (accumulate) {
-    inverseBinMajor<N, true, 1><<<dim3(Jp / SL, I), dim3(kT), 0, s>>>(SC, I, Jp, out, scale);
-  } else {
-    inverseBinMajor<N, false, 1><<<dim3(Jp / SL, I), dim3(kT), 0, s>>>(SC, I, Jp, out, scale);
-  }
+      launchInverse(acc, groups, std::false_type{});
+  };
+  auto withGroups = [&](auto acc) {
+    if (pairedRuns)
+      withPairs(acc, std::integral_constant<int, 2>{});
+    else
+      withPairs(acc, std::integral_constant<int, 1>{});
+  };
+  if (accumulate)
+    withGroups(std::true_type{});
+  else
+    withGroups(std::false_type{});
   return launchStatus();
 }
 
@@ -754,8 +778,10 @@ size_t convWorkspaceBytes(int pass, int N, int B, int Cin, int Cout, int H, int 
   if ((long)B * ty * tx > (1L << 30)) return 0;
   int I, J, K;
   passDims(pass, B * ty * tx, Cin, Cout, &I, &J, &K);
-  size_t n = N == 8 ? workspaceFloat2<8>(I, J, K)
-                    : N == 16 ? workspaceFloat2<16>(I, J, K) : workspaceFloat2<32>(I, J, K);
+  const bool outTiled = pass != 2 && ty * tx > 1;  // the weight gradient is never tiled
+  size_t n = N == 8 ? workspaceFloat2<8>(I, J, K, outTiled)
+                    : N == 16 ? workspaceFloat2<16>(I, J, K, outTiled)
+                              : workspaceFloat2<32>(I, J, K, outTiled);
   return n * sizeof(float2);
 }
 

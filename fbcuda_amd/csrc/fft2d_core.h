@@ -229,7 +229,9 @@ __device__ __forceinline__ void columnPassInverse(const c32* plane, int l, c32 (
 // Two columns of results through a bounds-checked strided view (crop on store).
 // ACC adds the scaled result to what the view holds instead of replacing it;
 // ATOMIC does that with an atomic add (several workgroups contribute to one view).
-template <int N, bool ACC = false, bool ATOMIC = false>
+// PAIRS: the caller guarantees windowMovesAsPairs() for the view, so the lane's two
+// columns of a row are one 8-byte word, inside or outside the window together.
+template <int N, bool ACC = false, bool ATOMIC = false, bool PAIRS = false>
 __device__ __forceinline__ void storeColumnsWindow(float* dst, int sy, int sx, int h, int w, int padL,
                                                    int padU, int l, const c32 (&z0)[N / 2],
                                                    const c32 (&z1)[N / 2], float scale) {
@@ -238,6 +240,28 @@ __device__ __forceinline__ void storeColumnsWindow(float* dst, int sy, int sx, i
   // back so that both halves of a cache line reach L2 together.
   const int xa = 2 * l - padL, xb = xa + 1;
   const bool va = (unsigned)xa < (unsigned)w, vb = (unsigned)xb < (unsigned)w;
+  if constexpr (PAIRS) {
+    static_assert(!ATOMIC, "paired stores replace or add in place");
+    float2* pp = reinterpret_cast<float2*>(dst + xa);
+    const int sy2 = sy / 2;
+    staticFor<N>([&](auto yy) {
+      constexpr int y = decltype(yy)::value;
+      if ((unsigned)(y - padU) < (unsigned)h) {
+        const c32 a = z0[slot<N / 2>(y / 2)], c = z1[slot<N / 2>(y / 2)];
+        float2 v = float2{(y % 2 ? a.y : a.x) * scale, (y % 2 ? c.y : c.x) * scale};
+        float2* q = pp + (long)(y - padU) * sy2;
+        if (va) {
+          if constexpr (ACC) {
+            const float2 o = *q;
+            v.x += o.x;
+            v.y += o.y;
+          }
+          *q = v;
+        }
+      }
+    });
+    return;
+  }
   float* pa = dst + (long)xa * sx;
   float* pb = dst + (long)xb * sx;
   auto put = [&](float* q, float r) __attribute__((always_inline)) {
