@@ -376,22 +376,6 @@ def run_only(name, steps, warmup, F, synth, torch, dev):
             assert rc == 1
         _, t = timed(tiled, steps, warmup, torch)
         return {"only": name, "us": round(t * 1e6, 2)}
-    if name == "conv4":
-        # configs[4] updateOutput through the layer entry point (overlap-tiled pipeline)
-        x4 = synth.uniform((16, 32, 256, 256), seed=40, device=dev)
-        w4 = synth.normal((32, 32, 9, 9), seed=41, std=0.05, device=dev)
-        o4 = torch.empty((16, 32, 248, 248), device=dev)
-        ws4 = torch.empty(F.conv_workspace_image(0, 16, 32, 32, 256, 256, 9, 9, 32),
-                          dtype=torch.uint8, device=dev)
-        stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
-        v4 = (F.view(x4), F.view(w4), F.view(o4))
-
-        def layer():
-            rc = F.lib().fbfft_conv_fprop(ctypes.byref(v4[0]), ctypes.byref(v4[1]), ctypes.byref(v4[2]),
-                                          32, ctypes.c_void_p(ws4.data_ptr()), ws4.numel(), stream)
-            assert rc == 0
-        _, t = timed(layer, steps, warmup, torch)
-        return {"only": name, "us": round(t * 1e6, 2)}
     if name == "mm":
         A = synth.normal((128, 64, 17, 32, 2), seed=30, device=dev)
         Bm = synth.normal((192, 64, 17, 32, 2), seed=31, device=dev)
@@ -399,20 +383,39 @@ def run_only(name, steps, warmup, F, synth, torch, dev):
         mm = prepared("fbfft_transpose_mm", F, A, Bm, C, 0, 1, 0, ctypes.c_float(1.0 / 1024))
         _, t = timed(mm, steps, warmup, torch)
         return {"only": name, "us": round(t * 1e6, 2), "TFLOPs": round(6.845e9 / t / 1e12, 2)}
-    if name == "conv":
-        nb = int(os.environ.get("FBFFT_BENCH_CONV_B", "128"))  # profiling aid: other batch sizes
-        x = synth.normal((nb, 64, 27, 27), seed=30, device=dev)
-        w = synth.normal((192, 64, 5, 5), seed=31, std=0.02, device=dev)
-        out = torch.empty((nb, 192, 23, 23), device=dev)
-        ws = torch.empty(F.conv_fprop_workspace(nb, 64, 192, 32), dtype=torch.uint8, device=dev)
+    if name in ("conv", "conv_bprop", "conv_accgrad", "conv4", "conv4_bprop", "conv4_accgrad"):
+        # one pass of the convolution layer at configs[3] / configs[4] shapes
+        big = name.startswith("conv4")
+        pass_ = 1 if name.endswith("bprop") else 2 if name.endswith("accgrad") else 0
+        if big:
+            nb, cin, cout, hw, k = 16, 32, 32, 256, 9
+            x = synth.uniform((nb, cin, hw, hw), seed=40, device=dev)
+            w = synth.normal((cout, cin, k, k), seed=41, std=0.05, device=dev)
+        else:
+            nb = int(os.environ.get("FBFFT_BENCH_CONV_B", "128"))  # profiling aid: other batch sizes
+            cin, cout, hw, k = 64, 192, 27, 5
+            x = synth.normal((nb, cin, hw, hw), seed=30, device=dev)
+            w = synth.normal((cout, cin, k, k), seed=31, std=0.02, device=dev)
+        o = synth.normal((nb, cout, hw - k + 1, hw - k + 1), seed=32, device=dev)
+        ws = torch.empty(F.conv_workspace_image(pass_, nb, cin, cout, hw, hw, k, k, 32),
+                         dtype=torch.uint8, device=dev)
         stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
-        vx, vw, vo = F.view(x), F.view(w), F.view(out)
+        vx, vw, vo = F.view(x), F.view(w), F.view(o)
+        wsp, wsn = ctypes.c_void_p(ws.data_ptr()), ws.numel()
+        L = F.lib()
 
-        def conv():
-            rc = F.lib().fbfft_conv_fprop(ctypes.byref(vx), ctypes.byref(vw), ctypes.byref(vo), 32,
-                                          ctypes.c_void_p(ws.data_ptr()), ws.numel(), stream)
+        def layer():
+            if pass_ == 0:
+                rc = L.fbfft_conv_fprop(ctypes.byref(vx), ctypes.byref(vw), ctypes.byref(vo), 32,
+                                        wsp, wsn, stream)
+            elif pass_ == 1:
+                rc = L.fbfft_conv_bprop(ctypes.byref(vo), ctypes.byref(vw), ctypes.byref(vx), 32,
+                                        wsp, wsn, stream)
+            else:
+                rc = L.fbfft_conv_accgrad(ctypes.byref(vx), ctypes.byref(vo), ctypes.byref(vw), 32,
+                                          ctypes.c_float(1.0), 0, wsp, wsn, stream)
             assert rc == 0
-        _, t = timed(conv, steps, warmup, torch)
+        _, t = timed(layer, steps, warmup, torch)
         return {"only": name, "us": round(t * 1e6, 2)}
     conv_extras(F, synth, torch, dev, extra)
     return {"only": name, **extra}
@@ -430,7 +433,8 @@ def main():
     ap.add_argument("--no-extra", action="store_true", help="skip the informative extra configs")
     ap.add_argument("--only", default=None,
                     choices=["r2c32", "c2r32", "r2c64", "c2r64", "r2c128", "c2r128", "mm", "conv",
-                             "iterconv", "iter4", "conv4", "r2c1d", "c2r1d"],
+                             "conv_bprop", "conv_accgrad", "iterconv", "iter4", "conv4",
+                             "conv4_bprop", "conv4_accgrad", "r2c1d", "c2r1d"],
                     help="run just this workload --steps times (for rocprofv3) and print its timing")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="only run a plain 256 MiB device-to-device copy 20 times: the known-size "

@@ -47,10 +47,10 @@ namespace fbfft_amd {
 namespace {
 
 constexpr int kT = 256;
-#ifndef EXP_KTF
-#define EXP_KTF 256
-#endif
-constexpr int kTF = EXP_KTF;  // lanes of a transform workgroup
+// lanes of a transform workgroup: 16 planes of 32 x 32, so that a bin leaves or arrives as
+// a 128-byte run (measured at configs[3] / configs[4]: 128 lanes, 64-byte runs, +10 % /
+// +12 % per pass; 512 lanes, one workgroup per CU, +8 % / +6 %)
+constexpr int kTF = 256;
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
 template <int N>
@@ -239,7 +239,7 @@ __device__ __forceinline__ void forwardBinMajorBody(const ForwardJob& job, int w
 // LDS, and fly under the first run's transforms and stores.
 template <int N, bool ACC, int GROUPS, bool PAIRS>
 __global__ __launch_bounds__(kTF) void inverseBinMajor(const float2* Cs, int I, int Jp, PlaneSet out,
-                                                      float scale) {
+                                                       float scale, int splits, long splitStride) {
   using C = BMCfg<N>;
   constexpr int H = C::H, T = C::T, SLOTS = C::SLOTS, RS = C::RS, PSZ = C::PSZ;
   constexpr int PER = C::BINS / T;
@@ -259,6 +259,16 @@ __global__ __launch_bounds__(kTF) void inverseBinMajor(const float2* Cs, int I, 
       constexpr int u = decltype(uu)::value;
       in[u] = src[(bq + T * u) * binStride];
     });
+    // partial products of a reduction cut into ranges: added in range order
+    for (int sp2 = 1; sp2 < splits; ++sp2) {
+      src += splitStride;
+      staticFor<PER>([&](auto uu) {
+        constexpr int u = decltype(uu)::value;
+        const c32 v = src[(bq + T * u) * binStride];
+        in[u].x += v.x;
+        in[u].y += v.y;
+      });
+    }
   };
   auto park = [&](const c32 (&in)[PER]) __attribute__((always_inline)) {
     c32* dstp = lds + sp * PSZ;
@@ -330,6 +340,11 @@ struct GemmArgs {
   int IT, JT;       // tiles per bin
   int N;            // transform size: bins 0 and N/2 hold pairs of real values
   float invNorm;
+  // register kernels only: the reduction is cut into `splits` ranges of slicesPerSplit
+  // k-slices (blockIdx.y names the range); range s writes its partial product to
+  // C + s * splitStride and the inverse kernel adds the partials in range order
+  int splits, slicesPerSplit;
+  long splitStride;
 };
 
 // The k-slices go from HBM straight into LDS (global_load_lds, 16 bytes per lane,
@@ -480,44 +495,73 @@ __global__ __launch_bounds__(kT, TI == 128 ? 3 : 4) void binGemmDirect(GemmArgs 
   }
 }
 
-// The same product with no LDS and no barriers: a wave owns one 32 x 32 sub-tile and
-// loads exactly the operand values its own MFMA lanes supply - lane (r, h) of
-// v_mfma_f32_32x32x2_f32 supplies row / column r at k = h, so one 8-byte load per lane
-// fetches k-rows 2s and 2s+1 of 32 consecutive rows (two 256-byte runs per wave
-// instruction).  Slices of 8 k ride a ring of three register sets, two in flight while
-// one is multiplied.  The four waves of a workgroup are the 2 x 2 sub-tiles of a
-// 64 x 64 tile: they re-read each other's operands out of the CU's vector cache,
-// nothing else ties them together.
+// The same product with no LDS in the loop and no barriers there: a wave loads exactly
+// the operand values its own MFMA lanes supply - lane (r, h) of v_mfma_f32_32x32x2_f32
+// supplies row / column r at k = h, so one 8-byte load per lane fetches k-rows 2s and
+// 2s+1 of 32 consecutive rows (two 256-byte runs per wave instruction).  Slices of 8 k
+// ride a ring of three register sets, two in flight while one is multiplied; the
+// scheduling barriers keep each slice's loads ahead of the products of the slice two
+// before it (left alone the compiler sinks the loads below the products and then waits
+// for all of them at the top of the loop).
+template <class Slice, class Fetch, class Multiply>
+__device__ __forceinline__ void ringOfThree(int first, int step, int n, Fetch fetch,
+                                            Multiply multiply) {
+  // slices first, first + step, ...: n of them
+  if (n <= 0) return;
+  Slice s0, s1, s2;
+  fetch(s0, first);
+  fetch(s1, first + step * min(1, n - 1));
+  int sl = 0;
+  for (; sl + 3 <= n; sl += 3) {
+    fetch(s2, first + step * min(sl + 2, n - 1));
+    __builtin_amdgcn_sched_barrier(0);
+    multiply(s0);
+    __builtin_amdgcn_sched_barrier(0);
+    fetch(s0, first + step * min(sl + 3, n - 1));
+    __builtin_amdgcn_sched_barrier(0);
+    multiply(s1);
+    __builtin_amdgcn_sched_barrier(0);
+    fetch(s1, first + step * min(sl + 4, n - 1));
+    __builtin_amdgcn_sched_barrier(0);
+    multiply(s2);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  if (sl < n) {
+    multiply(s0);
+    if (sl + 1 < n) multiply(s1);
+  }
+}
+
+// Both sides short (up to 32 rows and 32 columns per bin, any K - the weight gradient
+// of a layer with few planes reduces over every image and window): one workgroup per
+// bin and range of the reduction; its four waves take every fourth k-slice each and
+// wave 0 adds the four 32 x 32 partial tiles in wave order (through LDS) before it
+// stores, so the result does not depend on timing.
 struct GemmSlice {
   float2 a[GK2 / 2], b[GK2 / 2];
 };
 
-__global__ __launch_bounds__(kT, 4) void binGemmRegs(GemmArgs g) {
+__global__ __launch_bounds__(kT, 4) void binGemmRegsSplitK(GemmArgs g) {
+  __shared__ float red[3][48][64];
   const int t = threadIdx.x;
   const int lane = t % 64, w = t / 64;
   const int r = lane % 32, h = lane / 32;
-  const int total = g.bins * g.IT * g.JT;
-  const int per = (total + 7) / 8;
-  const int logical = (blockIdx.x % 8) * per + blockIdx.x / 8;
-  if (logical >= total) return;
-  const int bin = logical / (g.IT * g.JT);
-  const int rem = logical % (g.IT * g.JT);
-  const int i0 = (rem / g.JT) * 64 + 32 * (w % 2), j0 = (rem % g.JT) * 64 + 32 * (w / 2);
-  if (i0 >= g.I || j0 >= g.Jp) return;  // sub-tile past the edge: nothing to compute
+  const int per = (g.bins + 7) / 8;
+  const int bin = (blockIdx.x % 8) * per + blockIdx.x / 8;
+  if (bin >= g.bins) return;
   const bool pairs = bin == 0 || 2 * bin == g.N;  // bins of real pairs: (ar br, ai bi)
   const float cross = pairs ? 0.f : 1.f;
 
   // operand columns beyond the padded arrays are clamped (they feed accumulators that
   // are never stored)
-  const float2* pa = g.A + ((long)bin * g.Kp + h) * g.Ip + min(i0 + r, g.Ip - 1);
-  const float2* pb = g.B + ((long)bin * g.Kp + h) * g.Jp + min(j0 + r, g.Jp - 1);
+  const float2* pa = g.A + ((long)bin * g.Kp + h) * g.Ip + min(r, g.Ip - 1);
+  const float2* pb = g.B + ((long)bin * g.Kp + h) * g.Jp + min(r, g.Jp - 1);
   const long sa = 2L * g.Ip, sb = 2L * g.Jp;  // two k-rows
 
   floatx16 k1, k2, k3;
 #pragma unroll
   for (int v = 0; v < 16; ++v) k1[v] = k2[v] = k3[v] = 0.f;
 
-  const int slices = g.Kp / GK2;
   auto fetch = [&](GemmSlice& s, int sl) __attribute__((always_inline)) {
     const float2* qa = pa + (long)sl * (GK2 / 2) * sa;
     const float2* qb = pb + (long)sl * (GK2 / 2) * sb;
@@ -538,42 +582,130 @@ __global__ __launch_bounds__(kT, 4) void binGemmRegs(GemmArgs g) {
       k3 = __builtin_amdgcn_mfma_f32_32x32x2f32(a.y, __builtin_fmaf(cross, b.x, -b.y), k3, 0, 0, 0);
     }
   };
-  GemmSlice s0, s1, s2;
-  fetch(s0, 0);
-  fetch(s1, min(1, slices - 1));
-  int sl = 0;
-  // the scheduling barriers keep each slice's loads ahead of the products of the slice
-  // two before it; left alone the compiler sinks the loads below the products and then
-  // waits for all of them at the top of the loop
-  for (; sl + 3 <= slices; sl += 3) {
-    fetch(s2, min(sl + 2, slices - 1));
-    __builtin_amdgcn_sched_barrier(0);
-    multiply(s0);
-    __builtin_amdgcn_sched_barrier(0);
-    fetch(s0, min(sl + 3, slices - 1));
-    __builtin_amdgcn_sched_barrier(0);
-    multiply(s1);
-    __builtin_amdgcn_sched_barrier(0);
-    fetch(s1, min(sl + 4, slices - 1));
-    __builtin_amdgcn_sched_barrier(0);
-    multiply(s2);
-    __builtin_amdgcn_sched_barrier(0);
-  }
-  if (sl < slices) {
-    multiply(s0);
-    if (sl + 1 < slices) multiply(s1);
-  }
+  const int slices = g.Kp / GK2;
+  const int rangeFirst = blockIdx.y * g.slicesPerSplit;
+  const int rangeEnd = min(rangeFirst + g.slicesPerSplit, slices);
+  // wave w takes slices w, w + 4, ... of the range: the workgroup reads one front
+  const int first = rangeFirst + w;
+  ringOfThree<GemmSlice>(first, 4, first < rangeEnd ? (rangeEnd - first + 3) / 4 : 0, fetch,
+                         multiply);
 
-  float2* Cb = g.C + (long)bin * g.I * g.Jp;
-  const int j = j0 + r;
+  if (w > 0) {
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      red[w - 1][v][lane] = k1[v];
+      red[w - 1][16 + v][lane] = k2[v];
+      red[w - 1][32 + v][lane] = k3[v];
+    }
+  }
+  __syncthreads();
+  if (w > 0) return;
+#pragma unroll
+  for (int u = 0; u < 3; ++u)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      k1[v] += red[u][v][lane];
+      k2[v] += red[u][16 + v][lane];
+      k3[v] += red[u][32 + v][lane];
+    }
+  float2* Cb = g.C + blockIdx.y * g.splitStride + (long)bin * g.I * g.Jp;
+  if (r < g.Jp) {
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      const int i = 8 * (v / 4) + 4 * h + v % 4;
+      if (i < g.I)
+        Cb[(long)i * g.Jp + r] =
+            pairs ? float2{k1[v] * g.invNorm, -k3[v] * g.invNorm}
+                  : float2{(k1[v] - k3[v]) * g.invNorm, (k1[v] + k2[v]) * g.invNorm};
+    }
+  }
+}
+
+// The register kernel for products with a short side (up to 32 rows of C per bin; the
+// host puts the short side on i): a wave owns 32 rows x 64 columns.  Lane (r, h) loads
+// 16 bytes of B per k-pair - columns j0 + 2r and j0 + 2r + 1 at k = 2s + h - which feed two
+// MFMA sub-tiles with interleaved columns, and stores the two results of a row side by
+// side as 16 bytes: half the memory instructions of two 32 x 32 sub-tiles, 512-byte runs,
+// and A (small, shared by every wave of the bin) is read once per 64 columns.  The four
+// waves of a workgroup take consecutive column blocks.
+struct GemmSliceWide {
+  float2 a[GK2 / 2];
+  float4 b[GK2 / 2];
+};
+
+__global__ __launch_bounds__(kT, 2) void binGemmRegsWide(GemmArgs g) {
+  const int t = threadIdx.x;
+  const int lane = t % 64, w = t / 64;
+  const int r = lane % 32, h = lane / 32;
+  // g.IT: 32-row blocks, g.JT: workgroups (4 x 64 columns) along j
+  const int total = g.bins * g.IT * g.JT;
+  const int per = (total + 7) / 8;
+  const int logical = (blockIdx.x % 8) * per + blockIdx.x / 8;
+  if (logical >= total) return;
+  const int bin = logical / (g.IT * g.JT);
+  const int rem = logical % (g.IT * g.JT);
+  const int i0 = (rem / g.JT) * 32, j0 = ((rem % g.JT) * 4 + w) * 64;
+  if (j0 >= g.Jp) return;
+  const bool pairs = bin == 0 || 2 * bin == g.N;  // bins of real pairs: (ar br, ai bi)
+  const float cross = pairs ? 0.f : 1.f;
+
+  // operand columns beyond the padded arrays are clamped (they feed accumulators that
+  // are never stored); Jp is even and rows of B and C start on 16-byte boundaries
+  const float2* pa = g.A + ((long)bin * g.Kp + h) * g.Ip + min(i0 + r, g.Ip - 1);
+  const float2* pb = g.B + ((long)bin * g.Kp + h) * g.Jp + min(j0 + 2 * r, g.Jp - 2);
+  const long sa = 2L * g.Ip, sb = 2L * g.Jp;  // two k-rows
+
+  floatx16 k1[2], k2[2], k3[2];
+#pragma unroll
+  for (int q = 0; q < 2; ++q)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) k1[q][v] = k2[q][v] = k3[q][v] = 0.f;
+
+  auto fetch = [&](GemmSliceWide& s, int sl) __attribute__((always_inline)) {
+    const float2* qa = pa + (long)sl * (GK2 / 2) * sa;
+    const float2* qb = pb + (long)sl * (GK2 / 2) * sb;
+#pragma unroll
+    for (int u = 0; u < GK2 / 2; ++u) {
+      s.a[u] = qa[u * sa];
+      s.b[u] = *reinterpret_cast<const float4*>(qb + u * sb);
+    }
+  };
+  // a conj(b) = (k1 - k3) + i (k1 + k2) with k1 = (ar + ai) br, k2 = -ar (br + bi),
+  // k3 = ai (br - bi)
+  auto multiply = [&](const GemmSliceWide& s) __attribute__((always_inline)) {
+#pragma unroll
+    for (int u = 0; u < GK2 / 2; ++u) {
+      const float2 a = s.a[u];
+      const float as = __builtin_fmaf(cross, a.y, a.x);
+      const float4 b = s.b[u];
+      k1[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(as, b.x, k1[0], 0, 0, 0);
+      k2[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a.x, -b.x - b.y, k2[0], 0, 0, 0);
+      k3[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a.y, __builtin_fmaf(cross, b.x, -b.y), k3[0], 0, 0, 0);
+      k1[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(as, b.z, k1[1], 0, 0, 0);
+      k2[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a.x, -b.z - b.w, k2[1], 0, 0, 0);
+      k3[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a.y, __builtin_fmaf(cross, b.z, -b.w), k3[1], 0, 0, 0);
+    }
+  };
+  const int first = blockIdx.y * g.slicesPerSplit;
+  ringOfThree<GemmSliceWide>(first, 1, min(first + g.slicesPerSplit, g.Kp / GK2) - first, fetch,
+                             multiply);
+
+  float2* Cb = g.C + blockIdx.y * g.splitStride + (long)bin * g.I * g.Jp;
+  const int j = j0 + 2 * r;
   if (j < g.Jp) {
 #pragma unroll
     for (int v = 0; v < 16; ++v) {
       const int i = i0 + 8 * (v / 4) + 4 * h + v % 4;
-      if (i < g.I)
-        Cb[(long)i * g.Jp + j] =
-            pairs ? float2{k1[v] * g.invNorm, -k3[v] * g.invNorm}
-                  : float2{(k1[v] - k3[v]) * g.invNorm, (k1[v] + k2[v]) * g.invNorm};
+      if (i < g.I) {
+        float4 o;
+        if (pairs)
+          o = float4{k1[0][v] * g.invNorm, -k3[0][v] * g.invNorm, k1[1][v] * g.invNorm,
+                     -k3[1][v] * g.invNorm};
+        else
+          o = float4{(k1[0][v] - k3[0][v]) * g.invNorm, (k1[0][v] + k2[0][v]) * g.invNorm,
+                     (k1[1][v] - k3[1][v]) * g.invNorm, (k1[1][v] + k2[1][v]) * g.invNorm};
+        *reinterpret_cast<float4*>(Cb + (long)i * g.Jp + j) = o;
+      }
     }
   }
 }
@@ -589,7 +721,24 @@ inline int roundUp(int a, int b) { return (a + b - 1) / b * b; }
 // padded tile elements.
 inline bool swapRoles(int I, int J, bool outTiled) {
   if (outTiled) return true;
+  if (I <= 32 || J <= 32) return J < I;  // the register kernel takes the short side on i
   return (long)roundUp(J, GI) * roundUp(I, GJ2) < (long)roundUp(I, GI) * roundUp(J, GJ2);
+}
+
+// Ranges the register kernels cut the reduction into (I <= 32 after the roles are
+// set): enough of them for about two waves per SIMD, each wave keeping at least four
+// k-slices.  32-point transforms have 512 bins and never split (measured on the weight
+// gradient of configs[4], 32 x 32 per bin over 1936 windows, 2048 waves: two ranges
+// 337 -> 345 us, four 362 - the contraction moves at the rate its operands leave the
+// last-level cache, not at the rate waves ask); 8- and 16-point transforms have 32 and
+// 128 bins and would leave most of the chip idle on a long reduction.
+inline int gemmSplits(int bins, int I, int Jp, int Kp) {
+  if (I > 32) return 1;
+  const bool narrow = Jp <= 32;
+  const long waves = narrow ? 4L * bins : (long)bins * ceilDiv(Jp, 64);
+  const int want = (int)std::min<long>(16, ceilDiv(2048L, waves));
+  const int most = Kp / GK2 / (narrow ? 16 : 4);
+  return std::max(1, std::min(want, most));
 }
 
 template <int N>
@@ -597,7 +746,8 @@ size_t workspaceFloat2(int I, int J, int K, bool outTiled) {
   if (swapRoles(I, J, outTiled)) std::swap(I, J);
   const int SL = BMCfg<N>::SLOTS, bins = BMCfg<N>::BINS;
   const int Ip = roundUp(I, SL), Jp = roundUp(J, SL), Kp = roundUp(K, 8);
-  return (size_t)bins * ((size_t)Kp * Ip + (size_t)Kp * Jp + (size_t)I * Jp);
+  return (size_t)bins * ((size_t)Kp * Ip + (size_t)Kp * Jp +
+                         (size_t)gemmSplits(bins, I, Jp, Kp) * I * Jp);
 }
 
 // P[i][j] = scale * sum_k X[i][k] * op(Y[j][k]) for planes x(i,k), y(j,k) -> planes out(i,j);
@@ -668,12 +818,17 @@ int runPipeline(PlaneSet x, PlaneSet y, PlaneSet out, bool conjY, float scale, b
   // chip with fewer than eight workgroups per CU to balance (measured equal or
   // faster there: 84 -> 62 us for 64 x 192 x 128 per bin, 77 -> 69 us for 128 x 64 x 192)
   const bool small = roundUp(I, 64) < roundUp(I, GI) || (long)bins * ceilDiv(I, GI) * g.JT < 8 * 256;
-  // Up to 32 columns the LDS kernels' 64-column tiles would be half empty; the register
-  // kernel drops its idle sub-tiles (configs[4], 1936 x 32 x 32 per bin: 146 -> 139 us.
-  // At configs[3], 128 x 192 x 64 per bin, it is the slower one: 64 against 58 us.)
-  if (Jp <= 32 || I <= 32) {
-    g.IT = ceilDiv(I, 64);
-    binGemmRegs<<<dim3(roundUp(bins * g.IT * g.JT, 8)), dim3(kT), 0, s>>>(g);
+  // Up to 32 rows (the roles put a short side there) the LDS kernels' tiles would be
+  // half empty; the register kernel works on 32-row blocks
+  g.splits = gemmSplits(bins, I, Jp, Kp);
+  g.slicesPerSplit = ceilDiv(Kp / GK2, g.splits);
+  g.splitStride = (long)bins * I * Jp;
+  if (I <= 32 && Jp <= 32) {
+    binGemmRegsSplitK<<<dim3(roundUp(bins, 8), g.splits), dim3(kT), 0, s>>>(g);
+  } else if (I <= 32) {
+    g.IT = 1;
+    g.JT = ceilDiv(Jp, 256);
+    binGemmRegsWide<<<dim3(roundUp(bins * g.JT, 8), g.splits), dim3(kT), 0, s>>>(g);
   } else if (small) {
     g.IT = ceilDiv(I, 64);
     binGemmDirect<64><<<dim3(roundUp(bins * g.IT * g.JT, 8)), dim3(kT), 0, s>>>(g);
@@ -692,7 +847,7 @@ int runPipeline(PlaneSet x, PlaneSet y, PlaneSet out, bool conjY, float scale, b
   const bool po = movesAsPairs(out);
   auto launchInverse = [&](auto acc, auto groups, auto pairs) {
     inverseBinMajor<N, decltype(acc)::value, decltype(groups)::value, decltype(pairs)::value>
-        <<<igrid, dim3(kTF), 0, s>>>(SC, I, Jp, out, scale);
+        <<<igrid, dim3(kTF), 0, s>>>(SC, I, Jp, out, scale, g.splits, g.splitStride);
   };
   auto withPairs = [&](auto acc, auto groups) {
     if (po)

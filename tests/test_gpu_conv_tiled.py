@@ -31,6 +31,11 @@ SHAPES = [
     (16, 37, 37, 16, 1, 2, 2),      # filter as large as the transform: one output per tile
     (32, 70, 64, 7, 5, 18, 33),     # several plane groups per workgroup row
     (16, 31, 33, 4, 3, 3, 3),       # even filter: odd window origins (4-byte load path)
+    # few planes, many windows: the weight gradient is a short-sided product with a long
+    # reduction, which the register kernels cut into ranges (partials added by the inverse)
+    (8, 30, 30, 3, 24, 3, 5),       # both sides short: four ranges
+    (8, 30, 30, 3, 24, 3, 40),      # one side short: sixteen ranges
+    (16, 40, 40, 5, 40, 4, 6),      # 16-point windows: two ranges
 ]
 
 
