@@ -163,15 +163,12 @@ __device__ __forceinline__ void forwardBinMajorBody(const ForwardJob& job, int w
   c32* plane = lds + s * PSZ;
 
   auto load = [&](int r0, c32 (&z0)[H], c32 (&z1)[H]) __attribute__((always_inline)) {
+    // padding planes (row >= R, k >= K) take the window of an existing plane and load nothing
     const int row = r0 + s;
-    if (row < ps.R && k < ps.K) {
-      const PlaneWindow win = planeWindow(ps, row, k);
-      loadColumnsWindow<N, PAIRS>(win.p, ps.sy, ps.sx, win.h, win.w, win.padL, win.padU, l, z0,
-                                  z1);
-    } else {
-#pragma unroll
-      for (int j = 0; j < H; ++j) z0[j] = z1[j] = c32{0.f, 0.f};
-    }
+    const bool present = row < ps.R && k < ps.K;
+    const PlaneWindow win = planeWindow(ps, min(row, ps.R - 1), min(k, ps.K - 1));
+    loadColumnsWindow<N, PAIRS>(win.p, ps.sy, ps.sx, win.h, win.w, win.padL, win.padU, l, z0, z1,
+                                present);
   };
   // lanes: sp = t % SLOTS walks the run (consecutive rows), bq = t / SLOTS in [0, T)
   // walks bins: lane (sp, bq) stores columns x = bq and bq + T of every spectral row,
@@ -600,7 +597,7 @@ __global__ __launch_bounds__(kT, 4) void binGemmRegsSplitK(GemmArgs g) {
   }
   __syncthreads();
   if (w > 0) return;
-#pragma unroll
+#pragma unroll 1
   for (int u = 0; u < 3; ++u)
 #pragma unroll
     for (int v = 0; v < 16; ++v) {
@@ -729,9 +726,9 @@ inline bool swapRoles(int I, int J, bool outTiled) {
 // set): enough of them for about two waves per SIMD, each wave keeping at least four
 // k-slices.  32-point transforms have 512 bins and never split (measured on the weight
 // gradient of configs[4], 32 x 32 per bin over 1936 windows, 2048 waves: two ranges
-// 337 -> 345 us, four 362 - the contraction moves at the rate its operands leave the
-// last-level cache, not at the rate waves ask); 8- and 16-point transforms have 32 and
-// 128 bins and would leave most of the chip idle on a long reduction.
+// 337 -> 345 us, four 362: that contraction is not short of waves); 8- and 16-point
+// transforms have 32 and 128 bins and would leave most of the chip idle on a long
+// reduction.
 inline int gemmSplits(int bins, int I, int Jp, int Kp) {
   if (I > 32) return 1;
   const bool narrow = Jp <= 32;

@@ -43,35 +43,44 @@ __host__ __device__ __forceinline__ bool windowMovesAsPairs(const float* src, lo
   return sx == 1 && ((sy | padL | w) & 1) == 0 && (reinterpret_cast<uintptr_t>(src) & 7) == 0;
 }
 
+// present = false: the plane does not exist (padding of a plane group);
+// no row passes the window test, so nothing is loaded and the columns are zero.  (A branch
+// around the call with a zero fill on the other side makes the compiler merge the stores
+// of both sides into stores through a selected address, which parks the columns in
+// scratch memory.)
 template <int N, int PAIRS = 2>
-__device__ __forceinline__ void loadColumnsWindow(const float* src, int sy, int sx, int h, int w,
-                                                  int padL, int padU, int l, c32 (&z0)[N / 2],
-                                                  c32 (&z1)[N / 2]) {
+__device__ __forceinline__ void loadColumnsWindow(const float* src, int sy, int sx, int hWindow,
+                                                  int w, int padL, int padU, int l,
+                                                  c32 (&z0)[N / 2], c32 (&z1)[N / 2],
+                                                  bool present = true) {
   if constexpr (PAIRS == 2) {
     if (windowMovesAsPairs(src, sy, sx, w, padL))
-      loadColumnsWindow<N, 1>(src, sy, sx, h, w, padL, padU, l, z0, z1);
+      loadColumnsWindow<N, 1>(src, sy, sx, hWindow, w, padL, padU, l, z0, z1, present);
     else
-      loadColumnsWindow<N, 0>(src, sy, sx, h, w, padL, padU, l, z0, z1);
+      loadColumnsWindow<N, 0>(src, sy, sx, hWindow, w, padL, padU, l, z0, z1, present);
     return;
   }
   const int xa = 2 * l - padL, xb = xa + 1;
   const bool va = (unsigned)xa < (unsigned)w, vb = (unsigned)xb < (unsigned)w;
+  const int h = present ? hWindow : 0;  // rows that pass the window test
   const int yEnd = padU + h;
   // rows in batches of 8: a batch that lies wholly below the window (the same for
   // every lane) issues no loads - a 5 x 5 filter plane costs 16 loads, not 2N
   if constexpr (PAIRS == 1) {
     const float* pp = src + min(max(xa, 0), w - 2);
+    // (zeroed up front rather than in an else branch: with stores to the same elements
+    // on both sides of a branch the compiler merges them into stores through a selected
+    // address, and the elements then live in scratch memory)
     float2 r[N];
+    staticFor<N>([&](auto yy) { r[decltype(yy)::value] = float2{0.0f, 0.0f}; });
     staticFor<(N + 7) / 8>([&](auto bb) {
       constexpr int y0 = 8 * decltype(bb)::value;
       constexpr int y1 = y0 + 8 < N ? y0 + 8 : N;
       if (y0 < yEnd) {
         staticFor<y1 - y0>([&](auto yy) {
           constexpr int y = y0 + decltype(yy)::value;
-          r[y] = *reinterpret_cast<const float2*>(pp + (long)min(max(y - padU, 0), h - 1) * sy);
+          r[y] = *reinterpret_cast<const float2*>(pp + (long)min(max(y - padU, 0), hWindow - 1) * sy);
         });
-      } else {
-        staticFor<y1 - y0>([&](auto yy) { r[y0 + decltype(yy)::value] = float2{0.0f, 0.0f}; });
       }
     });
     staticFor<N / 2>([&](auto jj) {
@@ -85,21 +94,16 @@ __device__ __forceinline__ void loadColumnsWindow(const float* src, int sy, int 
     const float* pa = src + (long)min(max(xa, 0), w - 1) * sx;
     const float* pb = src + (long)min(max(xb, 0), w - 1) * sx;
     float ra[N], rb[N];
+    staticFor<N>([&](auto yy) { ra[decltype(yy)::value] = rb[decltype(yy)::value] = 0.0f; });
     staticFor<(N + 7) / 8>([&](auto bb) {
       constexpr int y0 = 8 * decltype(bb)::value;
       constexpr int y1 = y0 + 8 < N ? y0 + 8 : N;
       if (y0 < yEnd) {
         staticFor<y1 - y0>([&](auto yy) {
           constexpr int y = y0 + decltype(yy)::value;
-          const long oy = (long)min(max(y - padU, 0), h - 1) * sy;
+          const long oy = (long)min(max(y - padU, 0), hWindow - 1) * sy;
           ra[y] = pa[oy];
           rb[y] = pb[oy];
-        });
-      } else {
-        staticFor<y1 - y0>([&](auto yy) {
-          constexpr int y = y0 + decltype(yy)::value;
-          ra[y] = 0.0f;
-          rb[y] = 0.0f;
         });
       }
     });
