@@ -266,11 +266,14 @@ __device__ __forceinline__ void storeColumnsWindow(float* dst, int sy, int sx, i
     });
     return;
   }
-  float* pa = dst + (long)xa * sx;
-  float* pb = dst + (long)xb * sx;
-  auto put = [&](float* q, float r) __attribute__((always_inline)) {
+  // (the view is device memory; said explicitly because a pointer that comes out of a
+  // descriptor in memory is generic and would make these flat instructions)
+  typedef __attribute__((address_space(1))) float* GlobalPtr;
+  GlobalPtr pa = (GlobalPtr)(dst + (long)xa * sx);
+  GlobalPtr pb = (GlobalPtr)(dst + (long)xb * sx);
+  auto put = [&](GlobalPtr q, float r) __attribute__((always_inline)) {
     if constexpr (ATOMIC)
-      atomicAdd(q, r * scale);
+      atomicAdd((float*)q, r * scale);
     else if constexpr (ACC)
       *q += r * scale;
     else

@@ -60,7 +60,10 @@ struct PlaneRef {
 __device__ __forceinline__ PlaneRef tilePlane(const fbfft_tile& t, int n, int c, int batch) {
   PlaneRef r;
   r.valid = n < batch && n < t.size[0] && c < t.size[1];
-  r.p = t.data + (size_t)n * t.stride[0] + (size_t)c * t.stride[1];
+  // the plane pointer comes out of a descriptor in memory: say that it is device memory,
+  // or every access through it is a flat instruction
+  typedef __attribute__((address_space(1))) float* GlobalPtr;
+  r.p = (float*)(GlobalPtr)(t.data + (size_t)n * t.stride[0] + (size_t)c * t.stride[1]);
   r.sy = t.stride[2];
   r.sx = t.stride[3];
   r.h = t.size[2];
