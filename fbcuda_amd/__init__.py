@@ -49,7 +49,7 @@ EXPORTS = (
     "fbfft_c2c_2d_inverse_pass1", "fbfft_transpose_mm", "fbfft_transpose_mm_packed", "fbfft_iterated_conv", "fbfft_iterated_conv_ex",
     "fbfft_make_tiles",
     "fbfft_make_tiles_for_pass",
-    "fbfft_conv_workspace", "fbfft_conv_workspace_image", "fbfft_conv_fprop_workspace", "fbfft_conv_fprop", "fbfft_conv_bprop",
+    "fbfft_conv_choose_fft_size", "fbfft_conv_workspace", "fbfft_conv_workspace_image", "fbfft_conv_fprop_workspace", "fbfft_conv_fprop", "fbfft_conv_bprop",
     "fbfft_conv_accgrad", "fbfft_conv_fprop_static", "fbfft_error_string",
     "fbfft_twiddle_table",
 )
@@ -90,6 +90,7 @@ def lib():
         L.fbfft_conv_fprop.argtypes = [tp, tp, tp, ctypes.c_int, vp, ctypes.c_size_t, vp]
         L.fbfft_conv_workspace.argtypes = [ctypes.c_int] * 5
         L.fbfft_conv_workspace.restype = ctypes.c_size_t
+        L.fbfft_conv_choose_fft_size.argtypes = [ctypes.c_int] * 4
         L.fbfft_conv_workspace_image.argtypes = [ctypes.c_int] * 9
         L.fbfft_conv_workspace_image.restype = ctypes.c_size_t
         L.fbfft_conv_bprop.argtypes = [tp, tp, tp, ctypes.c_int, vp, ctypes.c_size_t, vp]
@@ -282,9 +283,15 @@ def conv_workspace(pass_, batch, cin, cout, fftSize):
     return lib().fbfft_conv_workspace(int(pass_), batch, cin, cout, fftSize)
 
 
+def conv_choose_fft_size(H, W, kH, kW):
+    """The transform size that fftSize = 0 stands for in the conv_* calls (8, 16 or 32;
+    0 if no size fits the filter)."""
+    return lib().fbfft_conv_choose_fft_size(H, W, kH, kW)
+
+
 def conv_workspace_image(pass_, batch, cin, cout, H, W, kH, kW, fftSize):
     """Workspace bytes of a pass for input extents H x W (images larger than the transform
-    are overlap-tiled when fftSize <= 32)."""
+    are overlap-tiled when fftSize <= 32; fftSize 0: the library's choice)."""
     return lib().fbfft_conv_workspace_image(int(pass_), batch, cin, cout, H, W, kH, kW, fftSize)
 
 

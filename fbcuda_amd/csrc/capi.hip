@@ -234,12 +234,18 @@ namespace {
 
 bool convSizeOk(int N) { return N == 8 || N == 16 || N == 32 || N == 64 || N == 128; }
 
+// fftSize 0 in the layer entry points: the library's choice for the layer's extents.
+int resolveFftSize(int N, int H, int W, int kH, int kW) {
+  return N == 0 ? fbfft_conv_choose_fft_size(H, W, kH, kW) : N;
+}
+
 // Shapes of one convolution layer: input [B][Cin][H][W], weight [Cout][Cin][kH][kW],
 // output [B][Cout][H-kH+1][W-kW+1], H, W <= N.
 int checkConvShapes(const fbfft_tensor* input, const fbfft_tensor* weight,
                     const fbfft_tensor* output, int N) {
   if (!okTensor(input, 4) || !okTensor(weight, 4) || !okTensor(output, 4))
     return FBFFT_UNSUPPORTED_DIMENSION;
+  if (N == 0) N = resolveFftSize(0, input->size[2], input->size[3], weight->size[2], weight->size[3]);
   if (!convSizeOk(N)) return FBFFT_UNSUPPORTED_SIZE;
   const int B = input->size[0], Cin = input->size[1], H = input->size[2], W = input->size[3];
   const int Cout = weight->size[0], kH = weight->size[2], kW = weight->size[3];
@@ -259,6 +265,7 @@ int convPass(int pass, const fbfft_tensor* input, const fbfft_tensor* weight,
   const int rc = checkConvShapes(input, weight, output, N);
   if (rc != FBFFT_SUCCESS) return rc;
   if (empty(input) || empty(weight) || empty(output)) return FBFFT_SUCCESS;
+  N = resolveFftSize(N, input->size[2], input->size[3], weight->size[2], weight->size[3]);
   const size_t need = fbfft_conv_workspace_image(pass, input->size[0], input->size[1],
                                                  weight->size[0], input->size[2], input->size[3],
                                                  weight->size[2], weight->size[3], N);
@@ -278,9 +285,30 @@ int convPass(int pass, const fbfft_tensor* input, const fbfft_tensor* weight,
 
 }  // namespace
 
+extern "C" int fbfft_conv_choose_fft_size(int H, int W, int kH, int kW) {
+  if (kH < 1 || kW < 1 || kH > H || kW > W) return 0;
+  // the transform whose windows hold the fewest spectrum values: windows x N^2; the
+  // larger transform on a tie (fewer rows and columns loaded twice).  64 and 128 are
+  // never chosen: their layers run plane-major spectra through transposeMM and
+  // measure slower than 32-point windows on every shape tried.
+  int best = 0;
+  long bestCost = 0;
+  for (int N = 8; N <= 32; N *= 2) {
+    if (kH > N || kW > N) continue;
+    const long ty = (H - kH + 1 + N - kH) / (N - kH + 1), tx = (W - kW + 1 + N - kW) / (N - kW + 1);
+    const long cost = ty * tx * N * N;
+    if (best == 0 || cost <= bestCost) {
+      best = N;
+      bestCost = cost;
+    }
+  }
+  return best;
+}
+
 extern "C" size_t fbfft_conv_workspace_image(int pass, int batch, int cin, int cout, int H, int W,
                                              int kH, int kW, int fftSize) {
   if (pass < 0 || pass > 2 || batch <= 0 || cin <= 0 || cout <= 0) return 0;
+  if (fftSize == 0) fftSize = fbfft_conv_choose_fft_size(H, W, kH, kW);
   if (!convSizeOk(fftSize)) return 0;
   if (kH < 1 || kW < 1 || kH > H || kW > W || kH > fftSize || kW > fftSize) return 0;
   if ((H > fftSize || W > fftSize) && fftSize > 32) return 0;

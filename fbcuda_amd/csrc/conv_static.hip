@@ -54,7 +54,9 @@ extern "C" int fbfft_conv_fprop_static(const fbfft_tensor* input, const fbfft_te
                                        fbfft_stream_t stream) {
   if (!input || !weight || !output || input->dim != 4 || weight->dim != 4 || output->dim != 4)
     return FBFFT_UNSUPPORTED_DIMENSION;
-  const size_t need = fbfft_conv_workspace(0, input->size[0], input->size[1], weight->size[0], fftSize);
+  const size_t need = fbfft_conv_workspace_image(0, input->size[0], input->size[1], weight->size[0],
+                                                 input->size[2], input->size[3], weight->size[2],
+                                                 weight->size[3], fftSize);
   // need == 0: empty or unsupported shapes; fbfft_conv_fprop sorts those out and
   // never touches the workspace
   if (need > (size_t)FBFFT_STATIC_SCRATCH_BYTES) return FBFFT_UNSUPPORTED_SIZE;

@@ -236,3 +236,35 @@ def test_iterated_conv_refuses_filters_larger_than_the_transform():
                                      ctypes.cast(outs, ctypes.c_void_p), F.view(w), 0,
                                      ctypes.c_float(1.0), 1, 1, None)
     assert rc == 0
+
+
+def test_conv_choose_fft_size():
+    """fftSize = 0 of the layer entry points: fewest spectrum values over the windows
+    (windows x N^2 for N in 8, 16, 32 that hold the filter), larger N on a tie."""
+    def brute(H, W, kH, kW):
+        best = (None, 0)
+        for N in (8, 16, 32):
+            if kH > N or kW > N:
+                continue
+            ty = -(-(H - kH + 1) // (N - kH + 1))
+            tx = -(-(W - kW + 1) // (N - kW + 1))
+            cost = ty * tx * N * N
+            if best[0] is None or cost <= best[0]:
+                best = (cost, N)
+        return best[1]
+    L = F.lib()
+    for (H, W, kH, kW) in [(27, 27, 5, 5), (256, 256, 9, 9), (60, 60, 5, 5), (8, 8, 3, 3),
+                           (12, 40, 3, 5), (16, 16, 1, 1), (100, 7, 7, 7), (33, 33, 17, 2),
+                           (9, 9, 9, 9), (500, 300, 32, 32)]:
+        assert L.fbfft_conv_choose_fft_size(H, W, kH, kW) == brute(H, W, kH, kW), (H, W, kH, kW)
+    assert L.fbfft_conv_choose_fft_size(27, 27, 5, 5) == 32      # configs[3]
+    assert L.fbfft_conv_choose_fft_size(256, 256, 9, 9) == 32    # configs[4]
+    assert L.fbfft_conv_choose_fft_size(8, 8, 3, 3) == 8
+    # no size holds the filter, or the filter is larger than the image
+    assert L.fbfft_conv_choose_fft_size(64, 64, 33, 3) == 0
+    assert L.fbfft_conv_choose_fft_size(4, 4, 5, 5) == 0
+    # the workspace of size 0 is the workspace of the chosen size
+    for p in range(3):
+        assert L.fbfft_conv_workspace_image(p, 4, 3, 5, 60, 60, 5, 5, 0) == \
+            L.fbfft_conv_workspace_image(p, 4, 3, 5, 60, 60, 5, 5, 32)
+    assert L.fbfft_conv_workspace_image(0, 4, 3, 5, 64, 64, 33, 3, 0) == 0

@@ -120,3 +120,30 @@ def test_config4_through_the_layer_entry_point(oracle):
     oh = out.cpu().numpy()
     got = oh[coords[:, 0], coords[:, 1], coords[:, 2], coords[:, 3]]
     assert rel(got, want) < TOL_CONV
+
+
+@pytest.mark.parametrize("H,W,k,want", [(60, 60, 5, 32), (14, 12, 3, 16), (8, 8, 3, 8)])
+def test_fft_size_zero_is_the_library_choice(oracle, H, W, k, want):
+    """fftSize = 0: the three passes run on fbfft_conv_choose_fft_size's transform and
+    give that transform's results bit for bit."""
+    d = dev()
+    Bn, Cin, Cout = 3, 4, 5
+    assert F.conv_choose_fft_size(H, W, k, k) == want
+    x = synth.uniform((Bn, Cin, H, W), seed=40, device=d)
+    w = synth.normal((Cout, Cin, k, k), seed=41, std=0.05, device=d)
+    g = synth.normal((Bn, Cout, H - k + 1, W - k + 1), seed=42, device=d)
+    res = []
+    for N in (0, want):
+        out, gi, gw = torch.empty_like(g), torch.empty_like(x), torch.empty_like(w)
+        assert F.conv_fprop(x, w, out, N, ws(0, Bn, Cin, Cout, H, W, k, N)) == F.Success
+        assert F.conv_bprop(g, w, gi, N, ws(1, Bn, Cin, Cout, H, W, k, N)) == F.Success
+        assert F.conv_accgrad(x, g, gw, N, ws(2, Bn, Cin, Cout, H, W, k, N)) == F.Success
+        torch.cuda.synchronize()
+        res.append((out, gi, gw))
+    for a, b in zip(*res):
+        assert torch.equal(a, b)
+    assert rel(res[0][0].cpu().numpy(), oracle.corr2d_valid(x.cpu().numpy(), w.cpu().numpy())) < TOL_CONV
+    out = torch.empty_like(g)
+    assert F.conv_fprop_static(x, w, out, 0) == F.Success
+    torch.cuda.synchronize()
+    assert torch.equal(out, res[0][0])
