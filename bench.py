@@ -206,6 +206,21 @@ def conv_extras(F, synth, torch, dev, extra):
         "traffic": profile_figure("conv_pipeline_configs3.md", "traffic_bytes_per_iteration"),
         "algorithmic_bytes": 77119488,
         "workload": "configs[3]: 128x64x27x27 * 192x64x5x5 -> 128x192x23x23, 32-point FFTs"}
+    # the same pass with the transform size left to the library (fftSize 0): configs[3]
+    # names 32-point transforms, so this is an extra, not the metric
+    auto = L.fbfft_conv_choose_fft_size(0, 128, 64, 192, 27, 27, 5, 5)
+    wsa = torch.empty(F.conv_workspace_image(0, 128, 64, 192, 27, 27, 5, 5, 0), dtype=torch.uint8,
+                      device=dev)
+    wspa, wsba = ctypes.c_void_p(wsa.data_ptr()), wsa.numel()
+
+    def conv_auto():
+        if L.fbfft_conv_fprop(ctypes.byref(vx), ctypes.byref(vw), ctypes.byref(vo), 0, wspa, wsba,
+                              stream) != 0:
+            raise RuntimeError("fbfft_conv_fprop failed")
+    _, t = timed(conv_auto, 200, 200, torch)
+    extra["fft_conv_configs3_library_choice_ms_per_iter"] = round(t * 1e3, 4)
+    extra["fft_conv_configs3_library_choice_fft_size"] = auto
+    del wsa
     # the other two passes of the same layer
     g = synth.normal((128, 192, 23, 23), seed=32, device=dev)
     gi, gw = torch.empty_like(x), torch.empty_like(w)
@@ -397,7 +412,8 @@ def run_only(name, steps, warmup, F, synth, torch, dev):
             x = synth.normal((nb, cin, hw, hw), seed=30, device=dev)
             w = synth.normal((cout, cin, k, k), seed=31, std=0.02, device=dev)
         o = synth.normal((nb, cout, hw - k + 1, hw - k + 1), seed=32, device=dev)
-        ws = torch.empty(F.conv_workspace_image(pass_, nb, cin, cout, hw, hw, k, k, 32),
+        fft = int(os.environ.get("FBFFT_BENCH_CONV_N", "32"))  # profiling aid: other transform sizes
+        ws = torch.empty(F.conv_workspace_image(pass_, nb, cin, cout, hw, hw, k, k, fft),
                          dtype=torch.uint8, device=dev)
         stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
         vx, vw, vo = F.view(x), F.view(w), F.view(o)
@@ -406,13 +422,13 @@ def run_only(name, steps, warmup, F, synth, torch, dev):
 
         def layer():
             if pass_ == 0:
-                rc = L.fbfft_conv_fprop(ctypes.byref(vx), ctypes.byref(vw), ctypes.byref(vo), 32,
+                rc = L.fbfft_conv_fprop(ctypes.byref(vx), ctypes.byref(vw), ctypes.byref(vo), fft,
                                         wsp, wsn, stream)
             elif pass_ == 1:
-                rc = L.fbfft_conv_bprop(ctypes.byref(vo), ctypes.byref(vw), ctypes.byref(vx), 32,
+                rc = L.fbfft_conv_bprop(ctypes.byref(vo), ctypes.byref(vw), ctypes.byref(vx), fft,
                                         wsp, wsn, stream)
             else:
-                rc = L.fbfft_conv_accgrad(ctypes.byref(vx), ctypes.byref(vo), ctypes.byref(vw), 32,
+                rc = L.fbfft_conv_accgrad(ctypes.byref(vx), ctypes.byref(vo), ctypes.byref(vw), fft,
                                           ctypes.c_float(1.0), 0, wsp, wsn, stream)
             assert rc == 0
         _, t = timed(layer, steps, warmup, torch)

@@ -90,7 +90,7 @@ def lib():
         L.fbfft_conv_fprop.argtypes = [tp, tp, tp, ctypes.c_int, vp, ctypes.c_size_t, vp]
         L.fbfft_conv_workspace.argtypes = [ctypes.c_int] * 5
         L.fbfft_conv_workspace.restype = ctypes.c_size_t
-        L.fbfft_conv_choose_fft_size.argtypes = [ctypes.c_int] * 4
+        L.fbfft_conv_choose_fft_size.argtypes = [ctypes.c_int] * 8
         L.fbfft_conv_workspace_image.argtypes = [ctypes.c_int] * 9
         L.fbfft_conv_workspace_image.restype = ctypes.c_size_t
         L.fbfft_conv_bprop.argtypes = [tp, tp, tp, ctypes.c_int, vp, ctypes.c_size_t, vp]
@@ -283,10 +283,10 @@ def conv_workspace(pass_, batch, cin, cout, fftSize):
     return lib().fbfft_conv_workspace(int(pass_), batch, cin, cout, fftSize)
 
 
-def conv_choose_fft_size(H, W, kH, kW):
-    """The transform size that fftSize = 0 stands for in the conv_* calls (8, 16 or 32;
-    0 if no size fits the filter)."""
-    return lib().fbfft_conv_choose_fft_size(H, W, kH, kW)
+def conv_choose_fft_size(pass_, batch, cin, cout, H, W, kH, kW):
+    """The transform size that fftSize = 0 stands for in the conv_* call of that pass
+    (8, 16 or 32; 0 if no size fits the filter)."""
+    return lib().fbfft_conv_choose_fft_size(int(pass_), batch, cin, cout, H, W, kH, kW)
 
 
 def conv_workspace_image(pass_, batch, cin, cout, H, W, kH, kW, fftSize):

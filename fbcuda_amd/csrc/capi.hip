@@ -234,18 +234,21 @@ namespace {
 
 bool convSizeOk(int N) { return N == 8 || N == 16 || N == 32 || N == 64 || N == 128; }
 
-// fftSize 0 in the layer entry points: the library's choice for the layer's extents.
-int resolveFftSize(int N, int H, int W, int kH, int kW) {
-  return N == 0 ? fbfft_conv_choose_fft_size(H, W, kH, kW) : N;
+// fftSize 0 in the layer entry points: the library's choice for the pass and the layer.
+int resolveFftSize(int N, int pass, const fbfft_tensor* input, const fbfft_tensor* weight) {
+  return N != 0 ? N
+                : fbfft_conv_choose_fft_size(pass, input->size[0], input->size[1], weight->size[0],
+                                             input->size[2], input->size[3], weight->size[2],
+                                             weight->size[3]);
 }
 
 // Shapes of one convolution layer: input [B][Cin][H][W], weight [Cout][Cin][kH][kW],
 // output [B][Cout][H-kH+1][W-kW+1], H, W <= N.
-int checkConvShapes(const fbfft_tensor* input, const fbfft_tensor* weight,
+int checkConvShapes(int pass, const fbfft_tensor* input, const fbfft_tensor* weight,
                     const fbfft_tensor* output, int N) {
   if (!okTensor(input, 4) || !okTensor(weight, 4) || !okTensor(output, 4))
     return FBFFT_UNSUPPORTED_DIMENSION;
-  if (N == 0) N = resolveFftSize(0, input->size[2], input->size[3], weight->size[2], weight->size[3]);
+  N = resolveFftSize(N, pass, input, weight);
   if (!convSizeOk(N)) return FBFFT_UNSUPPORTED_SIZE;
   const int B = input->size[0], Cin = input->size[1], H = input->size[2], W = input->size[3];
   const int Cout = weight->size[0], kH = weight->size[2], kW = weight->size[3];
@@ -262,10 +265,10 @@ int checkConvShapes(const fbfft_tensor* input, const fbfft_tensor* weight,
 int convPass(int pass, const fbfft_tensor* input, const fbfft_tensor* weight,
              const fbfft_tensor* output, int N, float scale, bool accumulate, void* workspace,
              size_t workspaceBytes, fbfft_stream_t stream) {
-  const int rc = checkConvShapes(input, weight, output, N);
+  const int rc = checkConvShapes(pass, input, weight, output, N);
   if (rc != FBFFT_SUCCESS) return rc;
   if (empty(input) || empty(weight) || empty(output)) return FBFFT_SUCCESS;
-  N = resolveFftSize(N, input->size[2], input->size[3], weight->size[2], weight->size[3]);
+  N = resolveFftSize(N, pass, input, weight);
   const size_t need = fbfft_conv_workspace_image(pass, input->size[0], input->size[1],
                                                  weight->size[0], input->size[2], input->size[3],
                                                  weight->size[2], weight->size[3], N);
@@ -285,18 +288,28 @@ int convPass(int pass, const fbfft_tensor* input, const fbfft_tensor* weight,
 
 }  // namespace
 
-extern "C" int fbfft_conv_choose_fft_size(int H, int W, int kH, int kW) {
+extern "C" int fbfft_conv_choose_fft_size(int pass, int batch, int cin, int cout, int H, int W,
+                                          int kH, int kW) {
+  if (pass < 0 || pass > 2 || batch <= 0 || cin <= 0 || cout <= 0) return 0;
   if (kH < 1 || kW < 1 || kH > H || kW > W) return 0;
-  // the transform whose windows hold the fewest spectrum values: windows x N^2; the
-  // larger transform on a tie (fewer rows and columns loaded twice).  64 and 128 are
-  // never chosen: their layers run plane-major spectra through transposeMM and
-  // measure slower than 32-point windows on every shape tried.
+  // What a pass costs follows the spectrum values it moves: N^2 for every window of the
+  // two image-sized tensors and for every filter plane.  The forward pass and the weight
+  // gradient cut the OUTPUT into (N-kH+1) x (N-kW+1) windows, the input gradient cuts the
+  // INPUT.  Smaller transforms run a little below the rate of 32-point ones (measured
+  // over nine layer shapes: 1.15 x per value at 16 points, 1.5 x at 8), and their weight
+  // gradients well below (1.5 x and 3 x: many windows make a long reduction over small
+  // tiles).  The larger transform on a tie.  64 and 128 are never chosen: their layers run
+  // plane-major spectra through transposeMM and measure slower than 32-point windows on
+  // every shape tried.
   int best = 0;
-  long bestCost = 0;
+  double bestCost = 0;
   for (int N = 8; N <= 32; N *= 2) {
     if (kH > N || kW > N) continue;
-    const long ty = (H - kH + 1 + N - kH) / (N - kH + 1), tx = (W - kW + 1 + N - kW) / (N - kW + 1);
-    const long cost = ty * tx * N * N;
+    const int spanY = pass == 1 ? H : H - kH + 1, spanX = pass == 1 ? W : W - kW + 1;
+    const double tiles = (double)((spanY + N - kH) / (N - kH + 1)) * ((spanX + N - kW) / (N - kW + 1));
+    const double values = (double)N * N * (tiles * batch * ((double)cin + cout) + (double)cin * cout);
+    const double rate = N == 32 ? 1.0 : N == 16 ? (pass == 2 ? 1.5 : 1.15) : (pass == 2 ? 3.0 : 1.5);
+    const double cost = values * rate;
     if (best == 0 || cost <= bestCost) {
       best = N;
       bestCost = cost;
@@ -308,7 +321,7 @@ extern "C" int fbfft_conv_choose_fft_size(int H, int W, int kH, int kW) {
 extern "C" size_t fbfft_conv_workspace_image(int pass, int batch, int cin, int cout, int H, int W,
                                              int kH, int kW, int fftSize) {
   if (pass < 0 || pass > 2 || batch <= 0 || cin <= 0 || cout <= 0) return 0;
-  if (fftSize == 0) fftSize = fbfft_conv_choose_fft_size(H, W, kH, kW);
+  if (fftSize == 0) fftSize = fbfft_conv_choose_fft_size(pass, batch, cin, cout, H, W, kH, kW);
   if (!convSizeOk(fftSize)) return 0;
   if (kH < 1 || kW < 1 || kH > H || kW > W || kH > fftSize || kW > fftSize) return 0;
   if ((H > fftSize || W > fftSize) && fftSize > 32) return 0;

@@ -217,14 +217,19 @@ size_t fbfft_make_tiles_for_pass(int pass, const fbfft_tensor* input, const fbff
  * 256-byte aligned; its contents need not survive between calls. */
 
 /* fftSize = 0 in fbfft_conv_workspace_image, fbfft_conv_fprop / bprop / accgrad and
- * fbfft_conv_fprop_static stands for fbfft_conv_choose_fft_size(H, W, kH, kW): the size
- * in {8, 16, 32} (at least kH and kW) whose windows hold the fewest spectrum values, the
- * larger one on a tie; 0 if the filter is larger than the image or than 32.  The
- * reference leaves the choice to its caller (the FFTSize template parameter of
- * fbfft/FFTIteratedConvolution.cuh:624); 64 and 128 are only taken when asked for - on
- * this hardware 32-point windows measure faster than a 64- or 128-point transform of
- * the whole image (60 x 60 images, 5 x 5 filters: 39 us against 74 us and 229 us). */
-int fbfft_conv_choose_fft_size(int H, int W, int kH, int kW);
+ * fbfft_conv_fprop_static stands for fbfft_conv_choose_fft_size(pass, ...): the size in
+ * {8, 16, 32} (at least kH and kW) that is expected to run the pass fastest - the one
+ * that moves the fewest spectrum values over its windows and filter planes, weighted by
+ * the measured rate of each size; 0 if the filter is larger than the image or than 32.
+ * The passes of one layer may get different sizes (configs[3]: 16 for the forward pass,
+ * 91 us against 102 us at 32; 32 for both gradients); every size computes the same
+ * convolution.  The reference leaves the choice to its caller (the FFTSize template
+ * parameter of fbfft/FFTIteratedConvolution.cuh:624); 64 and 128 are only taken when asked
+ * for - on this hardware 32-point windows measure faster than a 64- or 128-point
+ * transform of the whole image (60 x 60 images, 5 x 5 filters: 36 us against 74 us and
+ * 229 us). */
+int fbfft_conv_choose_fft_size(int pass, int batch, int cin, int cout, int H, int W, int kH,
+                               int kW);
 
 /* Bytes of workspace for pass 0 (fprop), 1 (bprop) or 2 (accgrad): the values of
  * FFTConvolutionPassFFI (fbfft/FFTIteratedConvolution.cuh:616-622).  0 when the

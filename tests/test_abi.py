@@ -239,32 +239,33 @@ def test_iterated_conv_refuses_filters_larger_than_the_transform():
 
 
 def test_conv_choose_fft_size():
-    """fftSize = 0 of the layer entry points: fewest spectrum values over the windows
-    (windows x N^2 for N in 8, 16, 32 that hold the filter), larger N on a tie."""
-    def brute(H, W, kH, kW):
-        best = (None, 0)
-        for N in (8, 16, 32):
-            if kH > N or kW > N:
-                continue
-            ty = -(-(H - kH + 1) // (N - kH + 1))
-            tx = -(-(W - kW + 1) // (N - kW + 1))
-            cost = ty * tx * N * N
-            if best[0] is None or cost <= best[0]:
-                best = (cost, N)
-        return best[1]
+    """fftSize = 0 of the layer entry points: the choices recorded next to the measurements
+    they came from (forward pass / input gradient / weight gradient, us per pass at
+    fftSize 8, 16, 32 on one MI355X), and the properties every choice has."""
     L = F.lib()
-    for (H, W, kH, kW) in [(27, 27, 5, 5), (256, 256, 9, 9), (60, 60, 5, 5), (8, 8, 3, 3),
-                           (12, 40, 3, 5), (16, 16, 1, 1), (100, 7, 7, 7), (33, 33, 17, 2),
-                           (9, 9, 9, 9), (500, 300, 32, 32)]:
-        assert L.fbfft_conv_choose_fft_size(H, W, kH, kW) == brute(H, W, kH, kW), (H, W, kH, kW)
-    assert L.fbfft_conv_choose_fft_size(27, 27, 5, 5) == 32      # configs[3]
-    assert L.fbfft_conv_choose_fft_size(256, 256, 9, 9) == 32    # configs[4]
-    assert L.fbfft_conv_choose_fft_size(8, 8, 3, 3) == 8
-    # no size holds the filter, or the filter is larger than the image
-    assert L.fbfft_conv_choose_fft_size(64, 64, 33, 3) == 0
-    assert L.fbfft_conv_choose_fft_size(4, 4, 5, 5) == 0
-    # the workspace of size 0 is the workspace of the chosen size
-    for p in range(3):
-        assert L.fbfft_conv_workspace_image(p, 4, 3, 5, 60, 60, 5, 5, 0) == \
-            L.fbfft_conv_workspace_image(p, 4, 3, 5, 60, 60, 5, 5, 32)
+    measured = [
+        # batch, cin, cout, H, k: chosen size per pass
+        ((128, 64, 192, 27, 5), (16, 32, 32)),    # configs[3]: 206/90/102, 257/210/109, 422/111/107
+        ((16, 32, 32, 256, 9), (32, 32, 32)),     # configs[4]: -/500/285, -/506/284, -/551/310
+        ((32, 32, 64, 60, 5), (32, 16, 32)),      # 68/45/36, 82/55/76, 124/76/55
+        ((128, 96, 256, 13, 3), (8, 16, 16)),     # 48/50/173, 96/58/186, 60/55/193
+        ((128, 256, 256, 13, 3), (8, 16, 16)),    # 87/95/354, 161/95/355, 97/93/371
+        ((32, 64, 64, 56, 3), (16, 16, 32)),      # 51/43/50, 59/43/50, 214/74/56
+    ]
+    for (B, cin, cout, H, k), want in measured:
+        got = tuple(L.fbfft_conv_choose_fft_size(p, B, cin, cout, H, H, k, k) for p in range(3))
+        assert got == want, ((B, cin, cout, H, k), got)
+    for (H, W, kH, kW) in [(27, 27, 5, 5), (8, 8, 3, 3), (12, 40, 3, 5), (16, 16, 1, 1),
+                           (100, 7, 7, 7), (33, 33, 17, 2), (9, 9, 9, 9), (500, 300, 32, 32)]:
+        for p in range(3):
+            N = L.fbfft_conv_choose_fft_size(p, 4, 3, 5, H, W, kH, kW)
+            assert N in (8, 16, 32) and N >= max(kH, kW), (p, H, W, kH, kW, N)
+            # the workspace of size 0 is the workspace of the chosen size
+            assert L.fbfft_conv_workspace_image(p, 4, 3, 5, H, W, kH, kW, 0) == \
+                L.fbfft_conv_workspace_image(p, 4, 3, 5, H, W, kH, kW, N) > 0
+    # no size holds the filter, the filter is larger than the image, bad pass or counts
+    assert L.fbfft_conv_choose_fft_size(0, 4, 3, 5, 64, 64, 33, 3) == 0
+    assert L.fbfft_conv_choose_fft_size(0, 4, 3, 5, 4, 4, 5, 5) == 0
+    assert L.fbfft_conv_choose_fft_size(3, 4, 3, 5, 27, 27, 5, 5) == 0
+    assert L.fbfft_conv_choose_fft_size(0, 0, 3, 5, 27, 27, 5, 5) == 0
     assert L.fbfft_conv_workspace_image(0, 4, 3, 5, 64, 64, 33, 3, 0) == 0

@@ -122,27 +122,31 @@ def test_config4_through_the_layer_entry_point(oracle):
     assert rel(got, want) < TOL_CONV
 
 
-@pytest.mark.parametrize("H,W,k,want", [(60, 60, 5, 32), (14, 12, 3, 16), (8, 8, 3, 8)])
-def test_fft_size_zero_is_the_library_choice(oracle, H, W, k, want):
-    """fftSize = 0: the three passes run on fbfft_conv_choose_fft_size's transform and
-    give that transform's results bit for bit."""
+@pytest.mark.parametrize("H,W,k", [(60, 60, 5), (14, 12, 3), (8, 8, 3), (27, 27, 5)])
+def test_fft_size_zero_is_the_library_choice(oracle, H, W, k):
+    """fftSize = 0: each pass runs on fbfft_conv_choose_fft_size's transform for that pass
+    and gives that transform's results bit for bit."""
     d = dev()
     Bn, Cin, Cout = 3, 4, 5
-    assert F.conv_choose_fft_size(H, W, k, k) == want
     x = synth.uniform((Bn, Cin, H, W), seed=40, device=d)
     w = synth.normal((Cout, Cin, k, k), seed=41, std=0.05, device=d)
     g = synth.normal((Bn, Cout, H - k + 1, W - k + 1), seed=42, device=d)
+    chosen = [F.conv_choose_fft_size(p, Bn, Cin, Cout, H, W, k, k) for p in range(3)]
+    assert all(N in (8, 16, 32) for N in chosen)
     res = []
-    for N in (0, want):
+    for sizes in ((0, 0, 0), chosen):
         out, gi, gw = torch.empty_like(g), torch.empty_like(x), torch.empty_like(w)
-        assert F.conv_fprop(x, w, out, N, ws(0, Bn, Cin, Cout, H, W, k, N)) == F.Success
-        assert F.conv_bprop(g, w, gi, N, ws(1, Bn, Cin, Cout, H, W, k, N)) == F.Success
-        assert F.conv_accgrad(x, g, gw, N, ws(2, Bn, Cin, Cout, H, W, k, N)) == F.Success
+        assert F.conv_fprop(x, w, out, sizes[0], ws(0, Bn, Cin, Cout, H, W, k, sizes[0])) == F.Success
+        assert F.conv_bprop(g, w, gi, sizes[1], ws(1, Bn, Cin, Cout, H, W, k, sizes[1])) == F.Success
+        assert F.conv_accgrad(x, g, gw, sizes[2], ws(2, Bn, Cin, Cout, H, W, k, sizes[2])) == F.Success
         torch.cuda.synchronize()
         res.append((out, gi, gw))
     for a, b in zip(*res):
         assert torch.equal(a, b)
-    assert rel(res[0][0].cpu().numpy(), oracle.corr2d_valid(x.cpu().numpy(), w.cpu().numpy())) < TOL_CONV
+    xh, wh, gh = x.cpu().numpy(), w.cpu().numpy(), g.cpu().numpy()
+    assert rel(res[0][0].cpu().numpy(), oracle.corr2d_valid(xh, wh)) < TOL_CONV
+    assert rel(res[0][1].cpu().numpy(), oracle.corr2d_grad_input(gh, wh, H, W)) < TOL_CONV
+    assert rel(res[0][2].cpu().numpy(), oracle.corr2d_grad_weight(xh, gh, k, k)) < TOL_CONV
     out = torch.empty_like(g)
     assert F.conv_fprop_static(x, w, out, 0) == F.Success
     torch.cuda.synchronize()
