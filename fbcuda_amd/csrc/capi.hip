@@ -297,7 +297,7 @@ extern "C" int fbfft_conv_choose_fft_size(int pass, int batch, int cin, int cout
   // gradient cut the OUTPUT into (N-kH+1) x (N-kW+1) windows, the input gradient cuts the
   // INPUT.  Smaller transforms run a little below the rate of 32-point ones (measured
   // over nine layer shapes: 1.15 x per value at 16 points, 1.5 x at 8), and their weight
-  // gradients well below (1.5 x and 3 x: many windows make a long reduction over small
+  // gradients further below (1.25 x and 2 x: many windows make a long reduction over small
   // tiles).  The larger transform on a tie.  64 and 128 are never chosen: their layers run
   // plane-major spectra through transposeMM and measure slower than 32-point windows on
   // every shape tried.
@@ -308,7 +308,7 @@ extern "C" int fbfft_conv_choose_fft_size(int pass, int batch, int cin, int cout
     const int spanY = pass == 1 ? H : H - kH + 1, spanX = pass == 1 ? W : W - kW + 1;
     const double tiles = (double)((spanY + N - kH) / (N - kH + 1)) * ((spanX + N - kW) / (N - kW + 1));
     const double values = (double)N * N * (tiles * batch * ((double)cin + cout) + (double)cin * cout);
-    const double rate = N == 32 ? 1.0 : N == 16 ? (pass == 2 ? 1.5 : 1.15) : (pass == 2 ? 3.0 : 1.5);
+    const double rate = N == 32 ? 1.0 : N == 16 ? (pass == 2 ? 1.25 : 1.15) : (pass == 2 ? 2.0 : 1.5);
     const double cost = values * rate;
     if (best == 0 || cost <= bestCost) {
       best = N;

@@ -394,8 +394,10 @@ __global__ __launch_bounds__(kT, TI == 128 ? 3 : 4) void binGemmDirect(GemmArgs 
   const bool pairs = bin == 0 || 2 * bin == g.N;
   const float cross = pairs ? 0.f : 1.f;
 
-  const float2* Ab = g.A + (long)bin * g.Kp * g.Ip;
-  const float2* Bb = g.B + (long)bin * g.Kp * g.Jp;
+  // this workgroup's range of the reduction (blockIdx.y; no range is empty)
+  const int sliceFirst = blockIdx.y * g.slicesPerSplit;
+  const float2* Ab = g.A + ((long)bin * g.Kp + (long)sliceFirst * GK2) * g.Ip;
+  const float2* Bb = g.B + ((long)bin * g.Kp + (long)sliceFirst * GK2) * g.Jp;
   // per-lane source columns, clamped into the padded arrays
   const int ia = min(i0 + 2 * (TI == 128 ? lane : lane % 32), g.Ip - 2);
   const int jb = min(j0 + 2 * (lane % 32), g.Jp - 2);
@@ -415,7 +417,7 @@ __global__ __launch_bounds__(kT, TI == 128 ? 3 : 4) void binGemmDirect(GemmArgs 
       k3[q][v] = 0.f;
     }
 
-  const int slices = g.Kp / GK2;
+  const int slices = min(g.slicesPerSplit, g.Kp / GK2 - sliceFirst);
   // wave w moves rows 2w, 2w+1 of A and rows 2w, 2w+1 of B of a slice: LOADS instructions
   auto issue = [&](Stage& st, int sl) __attribute__((always_inline)) {
     const int k0 = sl * GK2;
@@ -476,7 +478,7 @@ __global__ __launch_bounds__(kT, TI == 128 ? 3 : 4) void binGemmDirect(GemmArgs 
   }
   __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): nothing may land in LDS after this wave is gone
 
-  float2* Cb = g.C + (long)bin * g.I * g.Jp;
+  float2* Cb = g.C + blockIdx.y * g.splitStride + (long)bin * g.I * g.Jp;
 #pragma unroll
   for (int q = 0; q < NQ; ++q) {
     const int j = j0 + 32 * (cb + q) + r;
@@ -722,20 +724,62 @@ inline bool swapRoles(int I, int J, bool outTiled) {
   return (long)roundUp(J, GI) * roundUp(I, GJ2) < (long)roundUp(I, GI) * roundUp(J, GJ2);
 }
 
-// Ranges the register kernels cut the reduction into (I <= 32 after the roles are
-// set): enough of them for about two waves per SIMD, each wave keeping at least four
-// k-slices.  32-point transforms have 512 bins and never split (measured on the weight
-// gradient of configs[4], 32 x 32 per bin over 1936 windows, 2048 waves: two ranges
-// 337 -> 345 us, four 362: that contraction is not short of waves); 8- and 16-point
-// transforms have 32 and 128 bins and would leave most of the chip idle on a long
-// reduction.
-inline int gemmSplits(int bins, int I, int Jp, int Kp) {
-  if (I > 32) return 1;
-  const bool narrow = Jp <= 32;
-  const long waves = narrow ? 4L * bins : (long)bins * ceilDiv(Jp, 64);
-  const int want = (int)std::min<long>(16, ceilDiv(2048L, waves));
-  const int most = Kp / GK2 / (narrow ? 16 : 4);
-  return std::max(1, std::min(want, most));
+// Which contraction kernel runs a product, on which tiles, and into how many ranges the
+// reduction is cut (range s writes its partial product to C + s * splitStride and the
+// inverse kernel adds the partials in range order, so the result does not depend on
+// timing).  A short side (up to 32, which the roles put on i) takes the register kernels:
+// the LDS kernels' tiles would be half empty.  64-row tiles when they waste fewer rows,
+// or when 128-row tiles would leave the chip with fewer than eight workgroups per CU to
+// balance (measured equal or faster there: 84 -> 62 us for 64 x 192 x 128 per bin,
+// 77 -> 69 us for 128 x 64 x 192).  Ranges: when the tiles alone leave most of the chip
+// idle and the reduction is long - 8- and 16-point transforms have 32 and 128 bins, and a
+// weight gradient reduces over every image and window - up to 16 of them, enough for
+// about two waves per SIMD in the register kernels and one round of workgroups in the LDS
+// kernels, each keeping at least `minSlices` k-slices (weight gradient of configs[3] on
+// 8-point windows: 423 -> 238 us; 64 x 64 x 512 per bin on 16-point windows: 73 -> 63 us;
+// ranges of 8 slices cost 6 % where 16 slices are all there are).  32-point transforms on short sides
+// have 512 bins and never split (measured on the weight gradient of configs[4], 32 x 32
+// per bin over 1936 windows, 2048 waves: two ranges 337 -> 345 us, four 362: that
+// contraction is not short of waves).
+struct GemmPlan {
+  enum Kind { RegsSplitK, RegsWide, Direct64, Direct128 } kind;
+  int IT, JT;
+  int splits, slicesPerSplit;
+};
+
+inline GemmPlan planGemm(int bins, int I, int Jp, int Kp) {
+  GemmPlan p;
+  long waves, target;
+  int minSlices;
+  if (I <= 32 && Jp <= 32) {
+    p.kind = GemmPlan::RegsSplitK;
+    p.IT = p.JT = 1;
+    waves = 4L * bins;
+    target = 2048;
+    minSlices = 16;
+  } else if (I <= 32) {
+    p.kind = GemmPlan::RegsWide;
+    p.IT = 1;
+    p.JT = ceilDiv(Jp, 256);
+    waves = (long)bins * ceilDiv(Jp, 64);
+    target = 2048;
+    minSlices = 4;
+  } else {
+    p.JT = ceilDiv(Jp, GJ2);
+    const bool small =
+        roundUp(I, 64) < roundUp(I, GI) || (long)bins * ceilDiv(I, GI) * p.JT < 8 * 256;
+    p.kind = small ? GemmPlan::Direct64 : GemmPlan::Direct128;
+    p.IT = ceilDiv(I, small ? 64 : GI);
+    waves = 4L * bins * p.IT * p.JT;
+    target = 4096;
+    minSlices = 16;
+  }
+  const int slices = Kp / GK2;
+  const int want = (int)std::min<long>(16, ceilDiv(target, waves));
+  const int most = std::max(1, slices / minSlices);
+  p.slicesPerSplit = ceilDiv(slices, std::min(want, most));
+  p.splits = ceilDiv(slices, p.slicesPerSplit);  // no range is empty
+  return p;
 }
 
 template <int N>
@@ -744,7 +788,7 @@ size_t workspaceFloat2(int I, int J, int K, bool outTiled) {
   const int SL = BMCfg<N>::SLOTS, bins = BMCfg<N>::BINS;
   const int Ip = roundUp(I, SL), Jp = roundUp(J, SL), Kp = roundUp(K, 8);
   return (size_t)bins * ((size_t)Kp * Ip + (size_t)Kp * Jp +
-                         (size_t)gemmSplits(bins, I, Jp, Kp) * I * Jp);
+                         (size_t)planGemm(bins, I, Jp, Kp).splits * I * Jp);
 }
 
 // P[i][j] = scale * sum_k X[i][k] * op(Y[j][k]) for planes x(i,k), y(j,k) -> planes out(i,j);
@@ -809,29 +853,19 @@ int runPipeline(PlaneSet x, PlaneSet y, PlaneSet out, bool conjY, float scale, b
   g.Ip = Ip;
   g.Jp = Jp;
   g.Kp = Kp;
-  g.JT = ceilDiv(Jp, GJ2);
   g.invNorm = 1.0f / (float)(N * N);
-  // 64-row tiles when they waste fewer rows, or when 128-row tiles would leave the
-  // chip with fewer than eight workgroups per CU to balance (measured equal or
-  // faster there: 84 -> 62 us for 64 x 192 x 128 per bin, 77 -> 69 us for 128 x 64 x 192)
-  const bool small = roundUp(I, 64) < roundUp(I, GI) || (long)bins * ceilDiv(I, GI) * g.JT < 8 * 256;
-  // Up to 32 rows (the roles put a short side there) the LDS kernels' tiles would be
-  // half empty; the register kernel works on 32-row blocks
-  g.splits = gemmSplits(bins, I, Jp, Kp);
-  g.slicesPerSplit = ceilDiv(Kp / GK2, g.splits);
+  const GemmPlan plan = planGemm(bins, I, Jp, Kp);
+  g.IT = plan.IT;
+  g.JT = plan.JT;
+  g.splits = plan.splits;
+  g.slicesPerSplit = plan.slicesPerSplit;
   g.splitStride = (long)bins * I * Jp;
-  if (I <= 32 && Jp <= 32) {
-    binGemmRegsSplitK<<<dim3(roundUp(bins, 8), g.splits), dim3(kT), 0, s>>>(g);
-  } else if (I <= 32) {
-    g.IT = 1;
-    g.JT = ceilDiv(Jp, 256);
-    binGemmRegsWide<<<dim3(roundUp(bins * g.JT, 8), g.splits), dim3(kT), 0, s>>>(g);
-  } else if (small) {
-    g.IT = ceilDiv(I, 64);
-    binGemmDirect<64><<<dim3(roundUp(bins * g.IT * g.JT, 8)), dim3(kT), 0, s>>>(g);
-  } else {
-    g.IT = ceilDiv(I, GI);
-    binGemmDirect<GI><<<dim3(roundUp(bins * g.IT * g.JT, 8)), dim3(kT), 0, s>>>(g);
+  const dim3 ggrid(roundUp(bins * g.IT * g.JT, 8), g.splits);
+  switch (plan.kind) {
+    case GemmPlan::RegsSplitK: binGemmRegsSplitK<<<ggrid, dim3(kT), 0, s>>>(g); break;
+    case GemmPlan::RegsWide: binGemmRegsWide<<<ggrid, dim3(kT), 0, s>>>(g); break;
+    case GemmPlan::Direct64: binGemmDirect<64><<<ggrid, dim3(kT), 0, s>>>(g); break;
+    case GemmPlan::Direct128: binGemmDirect<GI><<<ggrid, dim3(kT), 0, s>>>(g); break;
   }
   // Two runs per workgroup pay when the paired launch still fills the chip for three
   // rounds or more (two workgroups are resident per CU): 112 -> 108 us at configs[4],

@@ -36,6 +36,7 @@ SHAPES = [
     (8, 30, 30, 3, 24, 3, 5),       # both sides short: four ranges
     (8, 30, 30, 3, 24, 3, 40),      # one side short: sixteen ranges
     (16, 40, 40, 5, 40, 4, 6),      # 16-point windows: two ranges
+    (8, 30, 30, 3, 24, 40, 48),     # no short side: the LDS kernel's reduction in four ranges
 ]
 
 
