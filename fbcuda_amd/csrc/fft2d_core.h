@@ -212,18 +212,30 @@ __device__ __forceinline__ void rowPassInPlace(c32* plane, int l) {
 // Column pass (inverse): reads packed rows of columns 2l, 2l+1, undoes the
 // real-input fix-up and runs the inverse N/2-point FFTs.  On return
 // z[slot<N/2>(j)] = (X[2j][x], X[2j+1][x]) * N*N for the two columns.
-template <int N>
+// SPLIT: the lane takes columns l and l + N/2 instead of 2l and 2l + 1 (two 8-byte LDS
+// reads per row instead of one 16-byte read), so that a store instruction of
+// storeColumnsWindow<..., SPLIT> writes neighbouring floats from neighbouring lanes.
+template <int N, bool SPLIT = false>
 __device__ __forceinline__ void columnPassInverse(const c32* plane, int l, c32 (&z0)[N / 2],
                                                   c32 (&z1)[N / 2]) {
   constexpr int H = N / 2, RS = PlaneCfg<N>::RS;
   c32 p0[H], p1[H];
-  const c32* src = plane + 2 * l;
-  staticFor<H>([&](auto rr) {
-    constexpr int r = decltype(rr)::value;
-    float4 v = ldsLoad4(src + r * RS);
-    p0[r] = c32{v.x, v.y};
-    p1[r] = c32{v.z, v.w};
-  });
+  if constexpr (SPLIT) {
+    const c32* src = plane + l;
+    staticFor<H>([&](auto rr) {
+      constexpr int r = decltype(rr)::value;
+      p0[r] = src[r * RS];
+      p1[r] = src[r * RS + H];
+    });
+  } else {
+    const c32* src = plane + 2 * l;
+    staticFor<H>([&](auto rr) {
+      constexpr int r = decltype(rr)::value;
+      float4 v = ldsLoad4(src + r * RS);
+      p0[r] = c32{v.x, v.y};
+      p1[r] = c32{v.z, v.w};
+    });
+  }
   realFixupInverse<H>(p0, z0);
   realFixupInverse<H>(p1, z1);
   difFFT<H, false>(z0);
@@ -235,14 +247,18 @@ __device__ __forceinline__ void columnPassInverse(const c32* plane, int l, c32 (
 // ATOMIC does that with an atomic add (several workgroups contribute to one view).
 // PAIRS: the caller guarantees windowMovesAsPairs() for the view, so the lane's two
 // columns of a row are one 8-byte word, inside or outside the window together.
-template <int N, bool ACC = false, bool ATOMIC = false, bool PAIRS = false>
+// SPLIT: z0 / z1 are columns l and l + N/2 (columnPassInverse<N, true>): each of a row's
+// two store instructions then writes a contiguous run per plane instead of every other
+// float.
+template <int N, bool ACC = false, bool ATOMIC = false, bool PAIRS = false, bool SPLIT = false>
 __device__ __forceinline__ void storeColumnsWindow(float* dst, int sy, int sx, int h, int w, int padL,
                                                    int padU, int l, const c32 (&z0)[N / 2],
                                                    const c32 (&z1)[N / 2], float scale) {
+  static_assert(!(PAIRS && SPLIT), "paired stores need neighbouring columns in one lane");
   // The column tests are per lane and the same for every row; the row test is
   // wave-uniform (a scalar branch).  The two columns of a row are stored back to
   // back so that both halves of a cache line reach L2 together.
-  const int xa = 2 * l - padL, xb = xa + 1;
+  const int xa = (SPLIT ? l : 2 * l) - padL, xb = xa + (SPLIT ? N / 2 : 1);
   const bool va = (unsigned)xa < (unsigned)w, vb = (unsigned)xb < (unsigned)w;
   if constexpr (PAIRS) {
     static_assert(!ATOMIC, "paired stores replace or add in place");
