@@ -167,8 +167,11 @@ __device__ __forceinline__ void forwardBinMajorBody(const ForwardJob& job, int w
     const int row = r0 + s;
     const bool present = row < ps.R && k < ps.K;
     const PlaneWindow win = planeWindow(ps, min(row, ps.R - 1), min(k, ps.K - 1));
-    loadColumnsWindow<N, PAIRS>(win.p, ps.sy, ps.sx, win.h, win.w, win.padL, win.padU, l, z0, z1,
-                                present);
+    // 4-byte loads (odd widths or strides): the lane takes columns l and l + N/2, so that
+    // a load instruction reads neighbouring floats (configs[3]: input gradient 108.0 ->
+    // 101.6 us, weight gradient 108.0 -> 104.1 us; forward pass unchanged)
+    loadColumnsWindow<N, PAIRS, PAIRS == 0>(win.p, ps.sy, ps.sx, win.h, win.w, win.padL, win.padU,
+                                            l, z0, z1, present);
   };
   // lanes: sp = t % SLOTS walks the run (consecutive rows), bq = t / SLOTS in [0, T)
   // walks bins: lane (sp, bq) stores columns x = bq and bq + T of every spectral row,
@@ -205,7 +208,7 @@ __device__ __forceinline__ void forwardBinMajorBody(const ForwardJob& job, int w
   const int ra = (wg % job.rowGroups) * GROUPS * SLOTS;
   c32 za0[H], za1[H];
   load(ra, za0, za1);
-  columnPassForward<N>(za0, za1, plane, l);
+  columnPassForward<N, PAIRS == 0>(za0, za1, plane, l);
   planeSync();  // the lanes of a plane sit in one wave
   if constexpr (GROUPS == 2) {
     const int rb = ra + SLOTS;
@@ -217,7 +220,7 @@ __device__ __forceinline__ void forwardBinMajorBody(const ForwardJob& job, int w
     copyOut(ra);
     if (second) {
       __syncthreads();  // every wave has copied the first run out of the plane buffers
-      columnPassForward<N>(zb0, zb1, plane, l);
+      columnPassForward<N, PAIRS == 0>(zb0, zb1, plane, l);
       planeSync();
       rowPassInPlace<N, true>(plane, l);
       __syncthreads();

@@ -48,11 +48,15 @@ __host__ __device__ __forceinline__ bool windowMovesAsPairs(const float* src, lo
 // around the call with a zero fill on the other side makes the compiler merge the stores
 // of both sides into stores through a selected address, which parks the columns in
 // scratch memory.)
-template <int N, int PAIRS = 2>
+// SPLIT (PAIRS = 0 only): the lane's columns are l and l + N/2 instead of 2l and 2l + 1, so
+// that a load instruction reads neighbouring floats into neighbouring lanes; goes with
+// columnPassForward<N, true>.
+template <int N, int PAIRS = 2, bool SPLIT = false>
 __device__ __forceinline__ void loadColumnsWindow(const float* src, int sy, int sx, int hWindow,
                                                   int w, int padL, int padU, int l,
                                                   c32 (&z0)[N / 2], c32 (&z1)[N / 2],
                                                   bool present = true) {
+  static_assert(!SPLIT || PAIRS == 0, "split columns are loaded one float at a time");
   if constexpr (PAIRS == 2) {
     if (windowMovesAsPairs(src, sy, sx, w, padL))
       loadColumnsWindow<N, 1>(src, sy, sx, hWindow, w, padL, padU, l, z0, z1, present);
@@ -60,7 +64,7 @@ __device__ __forceinline__ void loadColumnsWindow(const float* src, int sy, int 
       loadColumnsWindow<N, 0>(src, sy, sx, hWindow, w, padL, padU, l, z0, z1, present);
     return;
   }
-  const int xa = 2 * l - padL, xb = xa + 1;
+  const int xa = (SPLIT ? l : 2 * l) - padL, xb = xa + (SPLIT ? N / 2 : 1);
   const bool va = (unsigned)xa < (unsigned)w, vb = (unsigned)xb < (unsigned)w;
   const int h = present ? hWindow : 0;  // rows that pass the window test
   const int yEnd = padU + h;
@@ -174,7 +178,7 @@ __device__ __forceinline__ void loadColumnsWindowPerLane(const float* src, int s
 
 // Column pass (forward): N/2-point FFTs of the two packed columns, real-input
 // fix-up, packed rows written to the plane buffer.
-template <int N>
+template <int N, bool SPLIT = false>
 __device__ __forceinline__ void columnPassForward(c32 (&z0)[N / 2], c32 (&z1)[N / 2], c32* plane,
                                                   int l) {
   constexpr int H = N / 2, RS = PlaneCfg<N>::RS;
@@ -183,11 +187,20 @@ __device__ __forceinline__ void columnPassForward(c32 (&z0)[N / 2], c32 (&z1)[N 
   c32 p0[H], p1[H];
   realFixupForward<H>(z0, p0);
   realFixupForward<H>(z1, p1);
-  c32* dst = plane + 2 * l;
-  staticFor<H>([&](auto rr) {
-    constexpr int r = decltype(rr)::value;
-    ldsStore4(dst + r * RS, p0[r], p1[r]);
-  });
+  if constexpr (SPLIT) {  // columns l and l + N/2
+    c32* dst = plane + l;
+    staticFor<H>([&](auto rr) {
+      constexpr int r = decltype(rr)::value;
+      dst[r * RS] = p0[r];
+      dst[r * RS + H] = p1[r];
+    });
+  } else {
+    c32* dst = plane + 2 * l;
+    staticFor<H>([&](auto rr) {
+      constexpr int r = decltype(rr)::value;
+      ldsStore4(dst + r * RS, p0[r], p1[r]);
+    });
+  }
 }
 
 // Row pass: lane l transforms packed row l in place (natural order in and out).
