@@ -245,12 +245,12 @@ def test_conv_choose_fft_size():
     L = F.lib()
     measured = [
         # batch, cin, cout, H, k: chosen size per pass
-        ((128, 64, 192, 27, 5), (16, 32, 16)),    # configs[3]: 206/90/102, 257/210/109, 238/107/110
-        ((16, 32, 32, 256, 9), (32, 32, 32)),     # configs[4]: -/500/285, -/506/284, -/551/310
-        ((32, 32, 64, 60, 5), (32, 16, 32)),      # 68/45/36, 82/55/76, 124/76/55
-        ((128, 96, 256, 13, 3), (8, 16, 16)),     # 48/50/173, 96/58/186, 59/55/194
-        ((128, 256, 256, 13, 3), (8, 16, 16)),    # 87/95/354, 161/95/355, 101/96/372
-        ((32, 64, 64, 56, 3), (16, 16, 32)),      # 51/43/50, 59/43/50, 82/63/56
+        ((128, 64, 192, 27, 5), (16, 32, 16)),    # configs[3]: 196/92/102, 236/184/99, 226/104/104
+        ((16, 32, 32, 256, 9), (32, 32, 32)),     # configs[4]: -/499/285, -/506/283, -/549/310
+        ((32, 32, 64, 60, 5), (32, 16, 32)),      # 68/45/36, 81/55/76, 123/76/55
+        ((128, 96, 256, 13, 3), (8, 16, 16)),     # 46/50/168, 94/56/181, 58/53/186
+        ((128, 256, 256, 13, 3), (8, 16, 16)),    # 87/92/351, 161/92/356, 97/91/365
+        ((32, 64, 64, 56, 3), (16, 16, 32)),      # 51/43/50, 60/43/50, 82/60/56
     ]
     for (B, cin, cout, H, k), want in measured:
         got = tuple(L.fbfft_conv_choose_fft_size(p, B, cin, cout, H, H, k, k) for p in range(3))
