@@ -294,6 +294,20 @@ def conv_extras(F, synth, torch, dev, extra):
     _, t = timed(tiled, 30, 20, torch)
     extra["iterated_conv_configs4_ms_per_iter"] = round(t * 1e3, 4)
     extra["iterated_conv_configs4_direct_equiv_TFLOPs"] = round(163.3e9 / t / 1e12, 1)
+    # the same descriptors through a caller-owned workspace (fbfft_iterated_conv_ws)
+    wsd = torch.empty(F.iterated_conv_workspace(32, 0, 16, n, 32, 32), dtype=torch.uint8, device=dev)
+    wsdp, wsdb = ctypes.c_void_p(wsd.data_ptr()), wsd.numel()
+
+    def tiled_ws():
+        rc = L.fbfft_iterated_conv_ws(32, ctypes.c_void_p(ins.data_ptr()),
+                                      ctypes.c_void_p(outs.data_ptr()), ctypes.byref(vw4), 0,
+                                      ctypes.c_float(1.0), 16, n, wsdp, wsdb, stream)
+        if rc != 1:
+            raise RuntimeError("fbfft_iterated_conv_ws returned %d" % rc)
+    _, t = timed(tiled_ws, 60, 30, torch)
+    extra["iterated_conv_ws_configs4_ms_per_iter"] = round(t * 1e3, 4)
+    extra["iterated_conv_ws_configs4_direct_equiv_TFLOPs"] = round(163.3e9 / t / 1e12, 1)
+    del wsd
     # the same layer through the convolution-layer entry point: the 121 windows per image
     # ride through the bin-major pipeline (spectra in a workspace) instead of the fused kernel
     ws4 = torch.empty(F.conv_workspace_image(0, 16, 32, 32, 256, 256, 9, 9, 32), dtype=torch.uint8,
@@ -375,7 +389,7 @@ def run_only(name, steps, warmup, F, synth, torch, dev):
         return {"only": name, "us": round(t * 1e6, 2),
                 "GBps": round(b * (4 * n + 8 * (n // 2 + 1)) / t / 1e9, 1)}
     extra = {}
-    if name == "iter4":
+    if name in ("iter4", "iter4ws"):
         # configs[4] updateOutput through the fused tiled kernel only
         x4 = synth.uniform((16, 32, 256, 256), seed=40, device=dev)
         w4 = synth.normal((32, 32, 9, 9), seed=41, std=0.05, device=dev)
@@ -389,6 +403,18 @@ def run_only(name, steps, warmup, F, synth, torch, dev):
                                              ctypes.c_void_p(outs.data_ptr()), ctypes.byref(vw4), 0,
                                              ctypes.c_float(1.0), 16, n, stream)
             assert rc == 1
+        if name == "iter4ws":
+            # the same descriptors through a caller-owned workspace
+            wsd = torch.empty(F.iterated_conv_workspace(32, 0, 16, n, 32, 32), dtype=torch.uint8,
+                              device=dev)
+
+            def tiled():  # noqa: F811
+                rc = F.lib().fbfft_iterated_conv_ws(32, ctypes.c_void_p(ins.data_ptr()),
+                                                    ctypes.c_void_p(outs.data_ptr()),
+                                                    ctypes.byref(vw4), 0, ctypes.c_float(1.0), 16, n,
+                                                    ctypes.c_void_p(wsd.data_ptr()), wsd.numel(),
+                                                    stream)
+                assert rc == 1
         _, t = timed(tiled, steps, warmup, torch)
         return {"only": name, "us": round(t * 1e6, 2)}
     if name == "mm":
@@ -449,7 +475,7 @@ def main():
     ap.add_argument("--no-extra", action="store_true", help="skip the informative extra configs")
     ap.add_argument("--only", default=None,
                     choices=["r2c32", "c2r32", "r2c64", "c2r64", "r2c128", "c2r128", "mm", "conv",
-                             "conv_bprop", "conv_accgrad", "iterconv", "iter4", "conv4",
+                             "conv_bprop", "conv_accgrad", "iterconv", "iter4", "iter4ws", "conv4",
                              "conv4_bprop", "conv4_accgrad", "r2c1d", "c2r1d"],
                     help="run just this workload --steps times (for rocprofv3) and print its timing")
     ap.add_argument("--calibrate-copy", action="store_true",

@@ -47,6 +47,7 @@ _lib = None
 EXPORTS = (
     "fbfft_r2c_1d", "fbfft_c2r_1d", "fbfft_r2c_2d", "fbfft_c2c_2d_pass2", "fbfft_c2r_2d",
     "fbfft_c2c_2d_inverse_pass1", "fbfft_transpose_mm", "fbfft_transpose_mm_packed", "fbfft_iterated_conv", "fbfft_iterated_conv_ex",
+    "fbfft_iterated_conv_workspace", "fbfft_iterated_conv_ws",
     "fbfft_make_tiles",
     "fbfft_make_tiles_for_pass",
     "fbfft_conv_choose_fft_size", "fbfft_conv_workspace", "fbfft_conv_workspace_image", "fbfft_conv_fprop_workspace", "fbfft_conv_fprop", "fbfft_conv_bprop",
@@ -79,6 +80,11 @@ def lib():
                                           ctypes.c_int, ctypes.c_size_t, vp]
         L.fbfft_iterated_conv_ex.argtypes = [ctypes.c_int, vp, vp, tp, ctypes.c_int, ctypes.c_float,
                                              ctypes.c_int, ctypes.c_size_t, ctypes.c_uint, vp]
+        L.fbfft_iterated_conv_workspace.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int,
+                                                    ctypes.c_size_t, ctypes.c_int, ctypes.c_int]
+        L.fbfft_iterated_conv_workspace.restype = ctypes.c_size_t
+        L.fbfft_iterated_conv_ws.argtypes = [ctypes.c_int, vp, vp, tp, ctypes.c_int, ctypes.c_float,
+                                             ctypes.c_int, ctypes.c_size_t, vp, ctypes.c_size_t, vp]
         L.fbfft_make_tiles.argtypes = [tp, tp, ctypes.c_int, ctypes.c_int, ctypes.c_int, vp, vp,
                                        ctypes.c_size_t]
         L.fbfft_make_tiles.restype = ctypes.c_size_t
@@ -251,6 +257,28 @@ def FFTIteratedConvolution(fftSize, ins, outs, weight, pass_, scale, batchSize, 
                                       DETERMINISTIC if deterministic else 0, _stream(stream))
     if rc < 0:
         raise RuntimeError("fbfft_iterated_conv: %s" % error_string(-rc))
+    return rc == 1
+
+
+def iterated_conv_workspace(fftSize, pass_, batchSize, numTiles, cin, cout):
+    """Workspace bytes of FFTIteratedConvolution(..., workspace=...) for that pass."""
+    return lib().fbfft_iterated_conv_workspace(fftSize, int(pass_), int(batchSize), int(numTiles),
+                                               cin, cout)
+
+
+def FFTIteratedConvolutionWS(fftSize, ins, outs, weight, pass_, scale, batchSize, numTiles,
+                             workspace, stream=None):
+    """FFTIteratedConvolution on the same tile descriptors through a caller-owned workspace
+    (fbfft_iterated_conv_ws): the three kernels of the layer entry points instead of the
+    fused kernel.  Returns True if launched."""
+    _on_gpu(ins, outs, weight, workspace)
+    rc = lib().fbfft_iterated_conv_ws(fftSize, ctypes.c_void_p(ins.data_ptr()),
+                                      ctypes.c_void_p(outs.data_ptr()), view(weight), int(pass_),
+                                      float(scale), int(batchSize), int(numTiles),
+                                      ctypes.c_void_p(workspace.data_ptr()),
+                                      workspace.numel() * workspace.element_size(), _stream(stream))
+    if rc < 0:
+        raise RuntimeError("fbfft_iterated_conv_ws: %s" % error_string(-rc))
     return rc == 1
 
 

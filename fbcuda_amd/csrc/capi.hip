@@ -459,6 +459,34 @@ extern "C" size_t fbfft_make_tiles(const fbfft_tensor* input, const fbfft_tensor
                                    capacity);
 }
 
+extern "C" size_t fbfft_iterated_conv_workspace(int fftSize, int pass, int batchSize,
+                                               size_t numTiles, int cin, int cout) {
+  if (!(fftSize == 8 || fftSize == 16 || fftSize == 32) || pass < 0 || pass > 2) return 0;
+  if (batchSize <= 0 || numTiles == 0 || cin <= 0 || cout <= 0) return 0;
+  if (numTiles > (size_t)1 << 30) return 0;
+  return describedWorkspaceBytes(pass, fftSize, (long)numTiles * batchSize, cin, cout);
+}
+
+extern "C" int fbfft_iterated_conv_ws(int fftSize, const fbfft_tile* ins, const fbfft_tile* outs,
+                                      const fbfft_tensor* weight, int pass, float scale,
+                                      int batchSize, size_t numTiles, void* workspace,
+                                      size_t workspaceBytes, fbfft_stream_t stream) {
+  if (!okTensor(weight, 4) || !ins || !outs) return 0;
+  if (!(fftSize == 8 || fftSize == 16 || fftSize == 32) || pass < 0 || pass > 2) return 0;
+  if (weight->size[2] > fftSize || weight->size[3] > fftSize) return 0;
+  if (batchSize <= 0 || numTiles == 0 || weight->size[0] <= 0 || weight->size[1] <= 0)
+    return 1;  // nothing to do
+  const size_t need = fbfft_iterated_conv_workspace(fftSize, pass, batchSize, numTiles,
+                                                    weight->size[1], weight->size[0]);
+  if (need == 0) return 0;
+  if (!workspace || !aligned(workspace, 256) || workspaceBytes < need)
+    return -FBFFT_UNSUPPORTED_DIMENSION;
+  const int rc = launchDescribedConv(pass, fftSize, ins, outs, weight->data, weight->stride,
+                                     weight->size, scale, batchSize, (int)numTiles, workspace,
+                                     stream);
+  return rc == FBFFT_SUCCESS ? 1 : -rc;
+}
+
 extern "C" int fbfft_iterated_conv(int fftSize, const fbfft_tile* ins, const fbfft_tile* outs,
                                    const fbfft_tensor* weight, int pass, float scale,
                                    int batchSize, size_t numTiles, fbfft_stream_t stream) {

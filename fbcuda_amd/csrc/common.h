@@ -88,6 +88,10 @@ int launchTwoPass(int N, int mode, float* src, long s0, long s1, long s2, float*
 // pass 0 / 1 / 2 = forward, input gradient, weight gradient (x, y, out as in conv_pipeline.hip)
 // H, W: the layer's input extents (larger than N: overlap tiling, N <= 32 only)
 size_t convWorkspaceBytes(int pass, int N, int B, int Cin, int Cout, int H, int W, int kH, int kW);
+size_t describedWorkspaceBytes(int pass, int N, long rows, int Cin, int Cout);
+int launchDescribedConv(int pass, int N, const fbfft_tile* ins, const fbfft_tile* outs, float* weight,
+                        const int* wStride, const int* wSize, float scale, int batch, int numTiles,
+                        void* workspace, hipStream_t s);
 int launchConvPass(int pass, int N, float* x, const int* xStride, const int* xSize, float* y,
                    const int* yStride, const int* ySize, float* out, const int* outStride,
                    const int* outSize, float scale, bool accumulate, void* workspace,

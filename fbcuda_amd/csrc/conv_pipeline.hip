@@ -73,7 +73,11 @@ struct BMCfg {
 // window at (orgY + ty*stepY, orgX + tx*stepX) clipped to the image - rows and
 // columns clipped off above / left become the plane's padU / padL, so the window
 // keeps its place inside the FFT plane.  padU0 / padL0 shift every window further
-// (where a cropped result sits inside the inverse transform's plane).
+// (where a cropped result sits inside the inverse transform's plane).  Described
+// (FFTIteratedConvolution's interface, fbfft/FFTIteratedConvolution.cuh:71-88): one of
+// the two indices is the composite (image, tile), image-major, and every tile is a
+// descriptor in device memory - a [batch][planes][h][w] view with its own strides and
+// pads; the other index is the plane within the view.
 struct PlaneSet {
   float* base;
   long sRow, sK;
@@ -82,6 +86,9 @@ struct PlaneSet {
   int tiled;        // 0: plain, 1: row is the composite index, 2: k is
   int tilesY, tilesX, stepY, stepX, orgY, orgX, winH, winW;
   int padU0, padL0;
+  const fbfft_tile* tiles;  // described sets: the descriptors
+  int described;            // 0: no, 1: row is the composite (image, tile), 2: k is
+  int numTiles;             // tiles per image
 };
 
 // Orders the LDS accesses of one wave: what its lanes wrote before is what its lanes
@@ -97,12 +104,36 @@ __device__ __forceinline__ void planeSync() {
 struct PlaneWindow {
   float* p;
   int h, w, padL, padU;
+  int sy, sx;
+  bool valid;  // described sets: the view holds this image and plane and is not empty
 };
 
 __device__ __forceinline__ PlaneWindow planeWindow(const PlaneSet& ps, int row, int k) {
+  if (ps.described) {
+    const int comp = ps.described == 1 ? row : k, other = ps.described == 1 ? k : row;
+    // image-major: consecutive composites are consecutive tiles of one image - in a
+    // row-major tiling neighbours in memory, which is what 16 planes of a workgroup should
+    // be (tile-major, 16 images of one tile: 345 instead of 296 us at configs[4])
+    const fbfft_tile& d = ps.tiles[comp % ps.numTiles];
+    const int n = comp / ps.numTiles;
+    PlaneWindow win;
+    win.valid = n < d.size[0] && other < d.size[1] && d.size[2] > 0 && d.size[3] > 0;
+    // a plane the view does not hold takes the place of one it does, and loads nothing
+    // (no row passes the window test, and with padU = 0 no batch of rows is asked for)
+    typedef __attribute__((address_space(1))) float* GlobalPtr;
+    win.p = (float*)(GlobalPtr)(d.data + (long)min(n, max(d.size[0] - 1, 0)) * d.stride[0] +
+                                (long)min(other, max(d.size[1] - 1, 0)) * d.stride[1]);
+    win.h = max(d.size[2], 0);
+    win.w = max(d.size[3], 0);
+    win.padU = win.valid ? d.padU : 0;
+    win.padL = d.padL;
+    win.sy = d.stride[2];
+    win.sx = d.stride[3];
+    return win;
+  }
   if (ps.tiled == 0)
     return PlaneWindow{ps.base + (long)row * ps.sRow + (long)k * ps.sK, ps.h, ps.w, ps.padL0,
-                       ps.padU0};
+                       ps.padU0, ps.sy, ps.sx, true};
   const int comp = ps.tiled == 1 ? row : k, other = ps.tiled == 1 ? k : row;
   const long sImg = ps.tiled == 1 ? ps.sRow : ps.sK, sOther = ps.tiled == 1 ? ps.sK : ps.sRow;
   const int perImage = ps.tilesY * ps.tilesX;
@@ -115,6 +146,9 @@ __device__ __forceinline__ PlaneWindow planeWindow(const PlaneSet& ps, int row, 
   win.w = min(x0 + ps.winW, ps.w) - xa;
   win.padU = ps.padU0 + ya - y0;
   win.padL = ps.padL0 + xa - x0;
+  win.sy = ps.sy;
+  win.sx = ps.sx;
+  win.valid = true;
   return win;
 }
 
@@ -165,12 +199,14 @@ __device__ __forceinline__ void forwardBinMajorBody(const ForwardJob& job, int w
   auto load = [&](int r0, c32 (&z0)[H], c32 (&z1)[H]) __attribute__((always_inline)) {
     // padding planes (row >= R, k >= K) take the window of an existing plane and load nothing
     const int row = r0 + s;
-    const bool present = row < ps.R && k < ps.K;
     const PlaneWindow win = planeWindow(ps, min(row, ps.R - 1), min(k, ps.K - 1));
+    const bool present = row < ps.R && k < ps.K && win.valid;
     // 4-byte loads (odd widths or strides): the lane takes columns l and l + N/2, so that
     // a load instruction reads neighbouring floats (configs[3]: input gradient 108.0 ->
-    // 101.6 us, weight gradient 108.0 -> 104.1 us; forward pass unchanged)
-    loadColumnsWindow<N, PAIRS, PAIRS == 0>(win.p, ps.sy, ps.sx, win.h, win.w, win.padL, win.padU,
+    // 101.6 us, weight gradient 108.0 -> 104.1 us; forward pass unchanged).  PAIRS = 2
+    // (described sets: the windows are only known on the device) decides per plane
+    // between 8-byte and 4-byte loads of columns 2l and 2l + 1.
+    loadColumnsWindow<N, PAIRS, PAIRS == 0>(win.p, win.sy, win.sx, win.h, win.w, win.padL, win.padU,
                                             l, z0, z1, present);
   };
   // lanes: sp = t % SLOTS walks the run (consecutive rows), bq = t / SLOTS in [0, T)
@@ -237,7 +273,7 @@ __device__ __forceinline__ void forwardBinMajorBody(const ForwardJob& job, int w
 // A workgroup takes GROUPS (1 or 2) runs of SLOTS consecutive j of one i.  With two, the
 // second run's spectra are requested as soon as the first run's have been parked in
 // LDS, and fly under the first run's transforms and stores.
-template <int N, bool ACC, int GROUPS, bool PAIRS>
+template <int N, bool ACC, int GROUPS, int PAIRS>
 __global__ __launch_bounds__(kTF) void inverseBinMajor(const float2* Cs, int I, int Jp, PlaneSet out,
                                                        float scale, int splits, long splitStride) {
   using C = BMCfg<N>;
@@ -295,9 +331,11 @@ __global__ __launch_bounds__(kTF) void inverseBinMajor(const float2* Cs, int I, 
     rowPassInPlace<N, false>(plane, l);
     planeSync();
     c32 z0[H], z1[H];
-    // without 8-byte stores a lane takes columns l and l + N/2, so that each store
-    // instruction writes a contiguous run per plane (configs[3]: 102.4 -> 101.5 us)
-    columnPassInverse<N, !PAIRS>(plane, l, z0, z1);
+    // PAIRS = 0, no 8-byte stores: a lane takes columns l and l + N/2, so that each store
+    // instruction writes a contiguous run per plane (configs[3]: 102.4 -> 101.5 us).
+    // PAIRS = 2 (described sets): columns 2l and 2l + 1, 8-byte or 4-byte stores decided
+    // per plane.
+    columnPassInverse<N, PAIRS == 0>(plane, l, z0, z1);
     const int j = j0 + s;
     // (Parking the cropped planes in LDS and writing them out as 16-byte runs - one
     // contiguous stream for dense outputs, row quads for windows of a tiled image - was
@@ -305,8 +343,19 @@ __global__ __launch_bounds__(kTF) void inverseBinMajor(const float2* Cs, int I, 
     // configs[4]: the kernel waits on its own chain of phases, not on store requests.)
     if (j < out.K) {  // out.K: number of valid output planes along j
       const PlaneWindow win = planeWindow(out, i, j);
-      storeColumnsWindow<N, ACC, false, PAIRS, !PAIRS>(
-          win.p, out.sy, out.sx, win.h, win.w, win.padL, win.padU, l, z0, z1, scale);
+      if (win.valid) {
+        if constexpr (PAIRS == 2) {
+          if (windowMovesAsPairs(win.p, win.sy, win.sx, win.w, win.padL))
+            storeColumnsWindow<N, ACC, false, true, false>(win.p, win.sy, win.sx, win.h, win.w,
+                                                           win.padL, win.padU, l, z0, z1, scale);
+          else
+            storeColumnsWindow<N, ACC, false, false, false>(win.p, win.sy, win.sx, win.h, win.w,
+                                                            win.padL, win.padU, l, z0, z1, scale);
+        } else {
+          storeColumnsWindow<N, ACC, false, PAIRS == 1, PAIRS == 0>(
+              win.p, win.sy, win.sx, win.h, win.w, win.padL, win.padU, l, z0, z1, scale);
+        }
+      }
     }
   };
 
@@ -804,13 +853,14 @@ int runPipeline(PlaneSet x, PlaneSet y, PlaneSet out, bool conjY, float scale, b
   using C = BMCfg<N>;
   const int SL = C::SLOTS, bins = C::BINS;
   float xSign = 1.0f, ySign = conjY ? 1.0f : -1.0f;
-  if (swapRoles(x.R, y.R, out.tiled != 0)) {
+  if (swapRoles(x.R, y.R, out.tiled != 0 || out.described != 0)) {
     // G[j][i] = sum_k op(Y[j]) * conj(conj X[i])
     std::swap(x, y);
     xSign = conjY ? -1.0f : 1.0f;
     ySign = -1.0f;
     std::swap(out.sRow, out.sK);
     if (out.tiled) out.tiled = 3 - out.tiled;
+    if (out.described) out.described = 3 - out.described;
   }
   const int I = x.R, J = y.R, K = x.K;
   out.R = I;
@@ -820,10 +870,14 @@ int runPipeline(PlaneSet x, PlaneSet y, PlaneSet out, bool conjY, float scale, b
   float2* SB = SA + (size_t)bins * Kp * Ip;
   float2* SC = SB + (size_t)bins * Kp * Jp;
 
-  // every window of a set starts on an 8-byte boundary with an even width and pad
+  // 1: every window of a set starts on an 8-byte boundary with an even width and pad;
+  // 2: the windows are described on the device, each plane decides for itself; 0: 4 bytes
   auto movesAsPairs = [](const PlaneSet& p) {
+    if (p.described) return 2;
     return windowMovesAsPairs(p.base, p.sy, p.sx, p.w, p.padL0) && p.sRow % 2 == 0 &&
-           p.sK % 2 == 0 && (!p.tiled || ((p.stepX | p.orgX | p.winW) & 1) == 0);
+                   p.sK % 2 == 0 && (!p.tiled || ((p.stepX | p.orgX | p.winW) & 1) == 0)
+               ? 1
+               : 0;
   };
   // Two runs per workgroup pay once the halved launch still fills every CU several
   // times over (measured: 114.5 -> 109.8 us on 3936 workgroups, 29.9 -> 33.7 us on a
@@ -832,17 +886,24 @@ int runPipeline(PlaneSet x, PlaneSet y, PlaneSet out, bool conjY, float scale, b
   const ForwardJob ja{x, SA, Ip, Kp, xSign, two ? ceilDiv(Ip / SL, 2) : Ip / SL},
       jb{y, SB, Jp, Kp, ySign, two ? ceilDiv(Jp / SL, 2) : Jp / SL};
   const dim3 fgrid((unsigned)(ja.rowGroups + jb.rowGroups) * Kp);
-  const bool pa = movesAsPairs(x), pb = movesAsPairs(y);
+  const int pa = movesAsPairs(x), pb = movesAsPairs(y);
   auto launchForward = [&](auto groups) {
     constexpr int G = decltype(groups)::value;
-    if (pa && pb)
-      forwardBinMajor<N, 1, 1, G><<<fgrid, dim3(kTF), 0, s>>>(ja, jb);
-    else if (pa)
-      forwardBinMajor<N, 1, 0, G><<<fgrid, dim3(kTF), 0, s>>>(ja, jb);
-    else if (pb)
-      forwardBinMajor<N, 0, 1, G><<<fgrid, dim3(kTF), 0, s>>>(ja, jb);
+    auto withB = [&](auto modeA) {
+      constexpr int A = decltype(modeA)::value;
+      if (pb == 2)
+        forwardBinMajor<N, A, 2, G><<<fgrid, dim3(kTF), 0, s>>>(ja, jb);
+      else if (pb == 1)
+        forwardBinMajor<N, A, 1, G><<<fgrid, dim3(kTF), 0, s>>>(ja, jb);
+      else
+        forwardBinMajor<N, A, 0, G><<<fgrid, dim3(kTF), 0, s>>>(ja, jb);
+    };
+    if (pa == 2)
+      withB(std::integral_constant<int, 2>{});
+    else if (pa == 1)
+      withB(std::integral_constant<int, 1>{});
     else
-      forwardBinMajor<N, 0, 0, G><<<fgrid, dim3(kTF), 0, s>>>(ja, jb);
+      withB(std::integral_constant<int, 0>{});
   };
   if (two)
     launchForward(std::integral_constant<int, 2>{});
@@ -880,16 +941,18 @@ int runPipeline(PlaneSet x, PlaneSet y, PlaneSet out, bool conjY, float scale, b
   const dim3 igrid(pairedRuns ? ceilDiv(Jp / SL, 2) : Jp / SL, I);
   // windows whose rows start on 8-byte boundaries with an even width: a lane stores its
   // two columns of a row as one 8-byte word
-  const bool po = movesAsPairs(out);
+  const int po = movesAsPairs(out);
   auto launchInverse = [&](auto acc, auto groups, auto pairs) {
     inverseBinMajor<N, decltype(acc)::value, decltype(groups)::value, decltype(pairs)::value>
         <<<igrid, dim3(kTF), 0, s>>>(SC, I, Jp, out, scale, g.splits, g.splitStride);
   };
   auto withPairs = [&](auto acc, auto groups) {
-    if (po)
-      launchInverse(acc, groups, std::true_type{});
+    if (po == 2)
+      launchInverse(acc, groups, std::integral_constant<int, 2>{});
+    else if (po == 1)
+      launchInverse(acc, groups, std::integral_constant<int, 1>{});
     else
-      launchInverse(acc, groups, std::false_type{});
+      launchInverse(acc, groups, std::integral_constant<int, 0>{});
   };
   auto withGroups = [&](auto acc) {
     if (pairedRuns)
@@ -1031,6 +1094,63 @@ int launchConvPass(int pass, int N, float* x, const int* xStride, const int* xSi
     case 8: return runPass<8>(pass, px, py, po, scale, accumulate, ws, s);
     case 16: return runPass<16>(pass, px, py, po, scale, accumulate, ws, s);
     case 32: return runPass<32>(pass, px, py, po, scale, accumulate, ws, s);
+  }
+  return FBFFT_UNSUPPORTED_SIZE;
+}
+
+// FFTIteratedConvolution's operands - device arrays of tile descriptors - through the
+// same three kernels: tile t of ins / outs is a [batch][planes][h][w] view with its own
+// strides and pads, the (image, tile) pairs ride as rows (passes 0 and 1) or as
+// reduction steps (pass 2).  Roles as in iterated_conv.hip's table: pass 0
+// outs[t](n, f) = sum_c ins[t](n, c) * conj(weight(f, c)), pass 1 ins[t](n, c) =
+// sum_f outs[t](n, f) * weight(f, c), pass 2 weight(f, c) = scale * sum_(t, n)
+// ins[t](n, c) * conj(outs[t](n, f)); results land at (padU, padL) of the destination's
+// plane.  The descriptors are only read on the device.
+size_t describedWorkspaceBytes(int pass, int N, long rows, int Cin, int Cout) {
+  if (rows <= 0 || rows > (1L << 30)) return 0;
+  int I, J, K;
+  passDims(pass, (int)rows, Cin, Cout, &I, &J, &K);
+  const bool outTiled = pass != 2;
+  const size_t n = N == 8 ? workspaceFloat2<8>(I, J, K, outTiled)
+                          : N == 16 ? workspaceFloat2<16>(I, J, K, outTiled)
+                                    : workspaceFloat2<32>(I, J, K, outTiled);
+  return n * sizeof(float2);
+}
+
+int launchDescribedConv(int pass, int N, const fbfft_tile* ins, const fbfft_tile* outs, float* weight,
+                        const int* wStride, const int* wSize, float scale, int batch, int numTiles,
+                        void* workspace, hipStream_t s) {
+  const int Cout = wSize[0], Cin = wSize[1];
+  auto described = [&](const fbfft_tile* tiles, bool compositeIsRow, int planes) {
+    PlaneSet p{};
+    p.tiles = tiles;
+    p.described = compositeIsRow ? 1 : 2;
+    p.numTiles = numTiles;
+    (compositeIsRow ? p.R : p.K) = numTiles * batch;
+    (compositeIsRow ? p.K : p.R) = planes;
+    return p;
+  };
+  float* w = weight;
+  PlaneSet px, py, po;
+  if (pass == 0) {
+    px = described(ins, true, Cin);
+    py = planes(w, wStride, wSize, 0, 1);
+    po = described(outs, true, Cout);
+  } else if (pass == 1) {
+    px = described(outs, true, Cout);
+    py = planes(w, wStride, wSize, 1, 0);
+    po = described(ins, true, Cin);
+  } else {
+    px = described(ins, false, Cin);
+    py = described(outs, false, Cout);
+    po = planes(w, wStride, wSize, 1, 0);
+  }
+  float2* ws = static_cast<float2*>(workspace);
+  const float sc = pass == 2 ? scale : 1.0f;
+  switch (N) {
+    case 8: return runPass<8>(pass, px, py, po, sc, false, ws, s);
+    case 16: return runPass<16>(pass, px, py, po, sc, false, ws, s);
+    case 32: return runPass<32>(pass, px, py, po, sc, false, ws, s);
   }
   return FBFFT_UNSUPPORTED_SIZE;
 }

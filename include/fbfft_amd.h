@@ -167,6 +167,30 @@ int fbfft_iterated_conv_ex(int fftSize, const fbfft_tile* ins, const fbfft_tile*
                            const fbfft_tensor* weight, int pass, float scale, int batchSize,
                            size_t numTiles, unsigned flags, fbfft_stream_t stream);
 
+/* detail::FFTIteratedConvolution<FFTSize> (fbfft/FFTIteratedConvolution.cuh:624-755) for
+ * callers that can lend a workspace: the same operands - device arrays of tile
+ * descriptors, any tiling - and the same results as fbfft_iterated_conv (to rounding;
+ * the three passes of its table: outs[t] = sum_c ins[t] (*) weight, ins[t] = sum_f
+ * outs[t] (*) weight, weight = scale * sum_(t, n) ins[t] (*) outs[t]), computed by the
+ * three kernels of the convolution layer entry points instead of the fused kernel: each
+ * filter plane is transformed once per call rather than once per tile and image group,
+ * and the per-frequency products run on the matrix cores (configs[4]: 0.29 ms against
+ * 0.62 ms).  The weight gradient is reproducible bit for bit from run to run.
+ * workspace: device memory of fbfft_iterated_conv_workspace(fftSize, pass, batchSize,
+ * numTiles, cin, cout) bytes, 256-byte aligned; contents need not survive.  Returns as
+ * fbfft_iterated_conv: 1 launched, 0 nothing matched (pass, fftSize in {8, 16, 32},
+ * filter larger than the transform), a negative fbfft_error on a workspace that is
+ * missing, misaligned or too small (-FBFFT_UNSUPPORTED_DIMENSION) or a launch failure.
+ * Tiles are read on the device only; a tile whose view does not hold an image or plane
+ * (size[0] < batchSize, fewer planes than the filter) contributes zeros, as in the
+ * fused kernel. */
+size_t fbfft_iterated_conv_workspace(int fftSize, int pass, int batchSize, size_t numTiles,
+                                     int cin, int cout);
+int fbfft_iterated_conv_ws(int fftSize, const fbfft_tile* ins, const fbfft_tile* outs,
+                           const fbfft_tensor* weight, int pass, float scale, int batchSize,
+                           size_t numTiles, void* workspace, size_t workspaceBytes,
+                           fbfft_stream_t stream);
+
 /* Host-side builder of the tile descriptors FFTIteratedConvolution consumes; the
  * reference leaves this to its external caller (fbfft/FFTIteratedConvolution.cuh:
  * 71-88 declares the descriptor, :113-114 consumes ins[tile] / outs[tile]).

@@ -470,6 +470,29 @@ bool FFTIteratedConvolution(TiledDeviceTensor<float, 4>* ins, TiledDeviceTensor<
                                 s) == 1;
 }
 
+// The same call for callers that can lend a workspace (not in the reference's
+// signature): the same descriptors and results, computed by the kernels of the
+// convolution layer entry points instead of the fused kernel - about twice as fast at
+// configs[4] - with a weight gradient that is reproducible bit for bit; see
+// fbfft_iterated_conv_ws.  workspaceBytes >= iteratedConvolutionWorkspace<FFTSize>(...).
+template <int FFTSize>
+size_t iteratedConvolutionWorkspace(const DeviceTensor<float, 4>& weight, FFTConvolutionPassFFI pass,
+                                    int batchSize, size_t numTiles) {
+  return fbfft_iterated_conv_workspace(FFTSize, pass.pass, batchSize, numTiles, weight.getSize(1),
+                                       weight.getSize(0));
+}
+
+template <int FFTSize>
+bool FFTIteratedConvolution(TiledDeviceTensor<float, 4>* ins, TiledDeviceTensor<float, 4>* outs,
+                            const DeviceTensor<float, 4> weight, FFTConvolutionPassFFI pass,
+                            float scale, int batchSize, size_t numTiles, void* workspace,
+                            size_t workspaceBytes, fbfft_stream_t s) {
+  fbfft_tensor w = fbfft_amd_detail::describe(weight);
+  return fbfft_iterated_conv_ws(FFTSize, reinterpret_cast<const fbfft_tile*>(ins),
+                                reinterpret_cast<const fbfft_tile*>(outs), &w, pass.pass, scale,
+                                batchSize, numTiles, workspace, workspaceBytes, s) == 1;
+}
+
 // Host-side tile grid for FFTIteratedConvolution<FFTSize>: fills ins / outs (host
 // arrays of capacity descriptors) and returns the tile count; see
 // fbfft_make_tiles_for_pass.  FFT_UpdateGradInput needs its own grid (disjoint

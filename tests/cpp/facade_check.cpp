@@ -156,6 +156,17 @@ double convLayerError() {
     if (!fbfft::detail::FFTIteratedConvolution<N>(dins, douts, tw, pass, 1.0f, B, n, 0)) return 1;
     hipDeviceSynchronize();
     worst = std::max(worst, relL2(download(dtiled, out.size()), out));
+    // the same descriptors through a workspace
+    HIP_OK(hipMemset(dtiled, 0xff, out.size() * 4));
+    const size_t wsBytes = fbfft::detail::iteratedConvolutionWorkspace<N>(tw, pass, B, n);
+    if (wsBytes == 0) return 1;
+    void* ws;
+    HIP_OK(hipMalloc(&ws, wsBytes));
+    if (!fbfft::detail::FFTIteratedConvolution<N>(dins, douts, tw, pass, 1.0f, B, n, ws, wsBytes, 0))
+      return 1;
+    hipDeviceSynchronize();
+    worst = std::max(worst, relL2(download(dtiled, out.size()), out));
+    hipFree(ws);
     hipFree(dins);
     hipFree(douts);
   }
