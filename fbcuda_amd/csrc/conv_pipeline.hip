@@ -314,6 +314,10 @@ __global__ __launch_bounds__(kTF) void inverseBinMajor(const float2* Cs, int I, 
     });
   };
   auto transformAndStore = [&](int j0) __attribute__((always_inline)) {
+    // where the result goes: asked for up front, so that a described set's descriptor
+    // (device memory) arrives under the transforms instead of ahead of the stores
+    const int j = j0 + s;
+    const PlaneWindow win = planeWindow(out, i, min(j, out.K - 1));
     {  // virtual bins of row 0 back to the packed row: Q[x] = C0[x] + i CH[x],
        // Q[N-x] = conj(C0[x]) + i conj(CH[x]); lane 0 sorts the four real values into
        // Q[0] = (C0[0], CH[0]) and Q[N/2] = (C0[N/2], CH[N/2]).  The T lanes of a plane
@@ -336,13 +340,11 @@ __global__ __launch_bounds__(kTF) void inverseBinMajor(const float2* Cs, int I, 
     // PAIRS = 2 (described sets): columns 2l and 2l + 1, 8-byte or 4-byte stores decided
     // per plane.
     columnPassInverse<N, PAIRS == 0>(plane, l, z0, z1);
-    const int j = j0 + s;
     // (Parking the cropped planes in LDS and writing them out as 16-byte runs - one
     // contiguous stream for dense outputs, row quads for windows of a tiled image - was
     // measured and is slower, 35.9 -> 36.6 us at configs[3] and 112 -> 131 us at
     // configs[4]: the kernel waits on its own chain of phases, not on store requests.)
     if (j < out.K) {  // out.K: number of valid output planes along j
-      const PlaneWindow win = planeWindow(out, i, j);
       if (win.valid) {
         if constexpr (PAIRS == 2) {
           if (windowMovesAsPairs(win.p, win.sy, win.sx, win.w, win.padL))
