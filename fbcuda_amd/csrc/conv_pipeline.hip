@@ -19,8 +19,15 @@
 //      counters show A + B fetched
 //      from HBM exactly once (the tiles of a bin share an L2: workgroup ids are
 //      remapped per XCD) and C written once with coalesced stores.
+//      binGemmRegsWide / binGemmRegsSplitK: the same product without LDS for
+//      products with a side of up to 32 (planGemm picks kernel, tiles and the
+//      ranges a long reduction is cut into).
 //   3. inverseBinMajor:  C[bin][i][j] -> planes, gathering runs of SLOTS
 //      consecutive j per bin, inverse transform, crop on store.
+//
+// The planes of an operand are a PlaneSet: whole tensors, overlapping windows of
+// images larger than the transform (the layer entry points), or the tile
+// descriptors of FFTIteratedConvolution in device memory (fbfft_iterated_conv_ws).
 //
 // Spectral rows 0 and N/2 of a real plane are both Hermitian along kx, so their
 // 2 N complex values carry N complex worth of information; they travel as N
