@@ -107,3 +107,52 @@ def test_graph_capture_of_the_tiled_convolution():
         # partial gradients meet in atomic adds: equal to rounding, not bit for bit
         assert bool(torch.isfinite(got[2]).all())
         assert float((got[2] - gw).norm() / gw.norm()) < 1e-5
+
+
+def test_graph_capture_of_the_workspace_tiled_convolution_and_size_choice():
+    """fbfft_iterated_conv_ws (tile descriptors read on the device, contraction launched on
+    a two-dimensional grid) and the layer entry points with fftSize 0 under capture."""
+    d = dev()
+    x = synth.uniform((4, 6, 40, 56), seed=40, device=d)
+    w = synth.normal((5, 6, 9, 9), seed=41, std=0.05, device=d)
+    out = torch.empty((4, 5, 32, 48), device=d)
+    out0 = torch.empty_like(out)
+    g = synth.normal(tuple(out.shape), seed=42, device=d)
+    gi, gw = torch.empty_like(x), torch.empty_like(w)
+    ins, outs, n = F.make_tile_grid(x, out, 9, 9, 32)
+    gins, gouts, n2 = F.make_tile_grid(gi, g, 9, 9, 32, F.FFT_UpdateGradInput)
+    ains, aouts, n3 = F.make_tile_grid(x, g, 9, 9, 32)
+    wsd = [torch.empty(F.iterated_conv_workspace(32, p, 4, m, 6, 5), dtype=torch.uint8, device=d)
+           for p, m in ((0, n), (1, n2), (2, n3))]
+    ws0 = torch.empty(F.conv_workspace_image(0, 4, 6, 5, 40, 56, 9, 9, 0), dtype=torch.uint8, device=d)
+
+    def run():
+        assert F.FFTIteratedConvolutionWS(32, ins, outs, w, F.FFT_UpdateOutput, 1.0, 4, n, wsd[0])
+        assert F.FFTIteratedConvolutionWS(32, gins, gouts, w, F.FFT_UpdateGradInput, 1.0, 4, n2, wsd[1])
+        assert F.FFTIteratedConvolutionWS(32, ains, aouts, gw, F.FFT_AccGradParameters, 0.5, 4, n3,
+                                          wsd[2])
+        assert F.conv_fprop(x, w, out0, 0, ws0) == F.Success
+
+    stream = torch.cuda.Stream()
+    stream.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(stream):
+        run()
+        stream.synchronize()
+        with torch.cuda.graph(graph, stream=stream):
+            run()
+    torch.cuda.synchronize()
+    for rep in range(3):
+        x.copy_(synth.uniform(tuple(x.shape), seed=60 + rep, device=d))
+        for t in (out, out0, gi, gw):
+            t.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [t.clone() for t in (out, out0, gi, gw)]
+        run()
+        torch.cuda.synchronize()
+        for a, b in zip(got, (out, out0, gi, gw)):
+            assert bool(torch.isfinite(a).all())
+            assert torch.equal(a, b), "replay %d differs from the eager result" % rep
+        assert float((out - out0).norm() / out0.norm()) < 1e-5
