@@ -12,7 +12,7 @@
 //   1. forwardBinMajor:  planes -> S[bin][k][row]   (row = image / output plane)
 //      a 256-lane workgroup transforms SLOTS = 512/N planes with consecutive
 //      `row` and the same k and writes each bin as one contiguous run.
-//   2. binGemmDirect:    C[bin][i][j] = invNorm * sum_k A[bin][k][i] * conj(B[bin][k][j])
+//   2. binGemmDirect:    C[bin][i][j] = sum_k A[bin][k][i] * conj(B[bin][k][j])
 //      one workgroup = one bin x (128 x 64) or (64 x 64) tile; k-slices of A and B
 //      are contiguous in HBM and are copied verbatim into LDS by global_load_lds;
 //      4 waves of MFMA 32x32x2 sub-tiles, three real products per complex one;
@@ -402,7 +402,6 @@ struct GemmArgs {
   int bins, I, Ip, Jp, Kp;
   int IT, JT;       // tiles per bin
   int N;            // transform size: bins 0 and N/2 hold pairs of real values
-  float invNorm;
   // register kernels only: the reduction is cut into `splits` ranges of slicesPerSplit
   // k-slices (blockIdx.y names the range); range s writes its partial product to
   // C + s * splitStride and the inverse kernel adds the partials in range order
@@ -418,6 +417,32 @@ struct GemmArgs {
 // rows zeroed; rows / columns beyond Ip / Jp are clamped (they only feed
 // accumulators that are never stored).
 constexpr int GJ2 = 64, GK2 = 8;
+
+// A wave-uniform address, pinned in scalar registers: the empty statement keeps the
+// compiler from folding it into a lane's offset, so that "scalar base + 32-bit lane
+// offset" reaches the memory instruction as its two operands and costs no vector
+// arithmetic.
+template <class T>
+__device__ __forceinline__ T* scalarBase(T* p) {
+  asm volatile("" : "+s"(p));
+  return p;
+}
+
+// ... and a lane's 32-bit offset kept apart from it up to the instruction (otherwise its
+// widening to 64 bits is hoisted and the sum becomes a vector addition per access).
+// (By value: the copy costs a move per access.  Marking the long-lived register itself
+// instead saves the moves and measured 1.5 us slower on the weight gradient of a
+// 128 x 64 x 27 x 27 * 192 x 64 x 5 x 5 layer, the same elsewhere.)
+__device__ __forceinline__ unsigned laneOffset(unsigned o) {
+  asm volatile("" : "+v"(o));
+  return o;
+}
+
+// plain vectors in global memory (float2's members take a generic `this`)
+typedef float __attribute__((ext_vector_type(2))) PlainPair;
+typedef __attribute__((address_space(1))) PlainPair GlobalPair;
+typedef float __attribute__((ext_vector_type(4))) PlainQuad;
+typedef __attribute__((address_space(1))) PlainQuad GlobalQuad;
 
 __device__ __forceinline__ void loadToLds(const float2* src, float2* ldsWaveBase) {
   __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
@@ -444,7 +469,10 @@ __global__ __launch_bounds__(kT, TI == 128 ? 3 : 4) void binGemmDirect(GemmArgs 
   // loads still in flight into the other three
   __shared__ __align__(16) Stage stage0, stage1, stage2, stage3;
   const int t = threadIdx.x;
-  const int lane = t % 64, w = t / 64;
+  const int lane = t % 64;
+  // the wave's number in a scalar register: everything below that depends only on it
+  // (LDS destinations, row offsets of the loads and of the result) is scalar arithmetic
+  const int w = __builtin_amdgcn_readfirstlane(t / 64);
   const int r = lane % 32, h = lane / 32;
 
   const int total = g.bins * g.IT * g.JT;
@@ -484,16 +512,20 @@ __global__ __launch_bounds__(kT, TI == 128 ? 3 : 4) void binGemmDirect(GemmArgs 
     }
 
   const int slices = min(g.slicesPerSplit, g.Kp / GK2 - sliceFirst);
-  // wave w moves rows 2w, 2w+1 of A and rows 2w, 2w+1 of B of a slice: LOADS instructions
+  // wave w moves rows 2w, 2w+1 of A and rows 2w, 2w+1 of B of a slice: LOADS instructions.
+  // An address is a scalar base (slice and wave) plus a lane's 32-bit byte offset that
+  // never changes, so a step spends no vector instructions on addresses.
+  const unsigned laneA = (unsigned)((TI == 128 ? 0 : h * g.Ip) + ia) * (unsigned)sizeof(float2);
+  const unsigned laneB = (unsigned)(h * g.Jp + jb) * (unsigned)sizeof(float2);
+  const char* const waveA = (const char*)(Ab + (long)(2 * w) * g.Ip);
+  const char* const waveB = (const char*)(Bb + (long)(2 * w) * g.Jp);
+  const long sliceA = (long)GK2 * g.Ip * sizeof(float2), sliceB = (long)GK2 * g.Jp * sizeof(float2);
   auto issue = [&](Stage& st, int sl) __attribute__((always_inline)) {
-    const int k0 = sl * GK2;
-    if constexpr (TI == 128) {
-      loadToLds(Ab + (long)(k0 + 2 * w) * g.Ip + ia, &st.A[2 * w][0]);
-      loadToLds(Ab + (long)(k0 + 2 * w + 1) * g.Ip + ia, &st.A[2 * w + 1][0]);
-    } else {
-      loadToLds(Ab + (long)(k0 + 2 * w + h) * g.Ip + ia, &st.A[2 * w][0]);
-    }
-    loadToLds(Bb + (long)(k0 + 2 * w + h) * g.Jp + jb, &st.B[2 * w][0]);
+    loadToLds((const float2*)(scalarBase(waveA + sl * sliceA) + laneOffset(laneA)), &st.A[2 * w][0]);
+    if constexpr (TI == 128)
+      loadToLds((const float2*)(scalarBase(waveA + sl * sliceA + g.Ip * sizeof(float2)) + laneOffset(laneA)),
+                &st.A[2 * w + 1][0]);
+    loadToLds((const float2*)(scalarBase(waveB + sl * sliceB) + laneOffset(laneB)), &st.B[2 * w][0]);
   };
 
   // One slice: wait for it, let everybody see it, request the slice three ahead into
@@ -549,7 +581,37 @@ __global__ __launch_bounds__(kT, TI == 128 ? 3 : 4) void binGemmDirect(GemmArgs 
   }
   __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): nothing may land in LDS after this wave is gone
 
+  // The sums leave unscaled; the inverse transform's factor carries 1 / N^2.
   float2* Cb = g.C + blockIdx.y * g.splitStride + (long)bin * g.I * g.Jp;
+  if (i0 + 32 * rb + 32 <= g.I && j0 + 32 * (cb + NQ) <= g.Jp) {
+    // the wave's whole block lies inside C: a scalar base per accumulator row plus the
+    // lane's fixed offset, no tests
+    const unsigned laneC = (unsigned)(4 * h * g.Jp + r) * (unsigned)sizeof(float2);
+    char* const waveC = (char*)(Cb + (long)(i0 + 32 * rb) * g.Jp + j0 + 32 * cb);
+    const long rowC = (long)g.Jp * sizeof(float2);
+    auto store = [&](auto realPairs) __attribute__((always_inline)) {
+#pragma unroll
+      for (int q = 0; q < NQ; ++q)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          // (global address space spelled out: behind the pinned base the compiler no
+          // longer sees where the pointer came from and would store through flat addresses)
+          typedef float __attribute__((ext_vector_type(2))) Pair;  // a plain vector: float2's assignment takes a generic `this`
+          auto* dst = (__attribute__((address_space(1))) Pair*)(
+              scalarBase(waveC + (8 * (v / 4) + v % 4) * rowC + q * 32 * (long)sizeof(float2)) +
+              laneOffset(laneC));
+          if constexpr (decltype(realPairs)::value)
+            *dst = Pair{k1[q][v], -k3[q][v]};
+          else
+            *dst = Pair{k1[q][v] - k3[q][v], k1[q][v] + k2[q][v]};
+        }
+    };
+    if (pairs)
+      store(std::true_type{});
+    else
+      store(std::false_type{});
+    return;
+  }
 #pragma unroll
   for (int q = 0; q < NQ; ++q) {
     const int j = j0 + 32 * (cb + q) + r;
@@ -558,9 +620,8 @@ __global__ __launch_bounds__(kT, TI == 128 ? 3 : 4) void binGemmDirect(GemmArgs 
     for (int v = 0; v < 16; ++v) {
       const int i = i0 + 32 * rb + 8 * (v / 4) + 4 * h + v % 4;
       if (i < g.I)
-        Cb[(long)i * g.Jp + j] =
-            pairs ? float2{k1[q][v] * g.invNorm, -k3[q][v] * g.invNorm}
-                  : float2{(k1[q][v] - k3[q][v]) * g.invNorm, (k1[q][v] + k2[q][v]) * g.invNorm};
+        Cb[(long)i * g.Jp + j] = pairs ? float2{k1[q][v], -k3[q][v]}
+                                       : float2{k1[q][v] - k3[q][v], k1[q][v] + k2[q][v]};
     }
   }
 }
@@ -634,7 +695,8 @@ struct GemmSlice {
 __global__ __launch_bounds__(kT, 4) void binGemmRegsSplitK(GemmArgs g) {
   __shared__ float red[3][48][64];
   const int t = threadIdx.x;
-  const int lane = t % 64, w = t / 64;
+  // (the wave's number in a scalar register: its slices and their addresses are scalar)
+  const int lane = t % 64, w = __builtin_amdgcn_readfirstlane(t / 64);
   const int r = lane % 32, h = lane / 32;
   const int per = (g.bins + 7) / 8;
   const int bin = (blockIdx.x % 8) * per + blockIdx.x / 8;
@@ -643,22 +705,26 @@ __global__ __launch_bounds__(kT, 4) void binGemmRegsSplitK(GemmArgs g) {
   const float cross = pairs ? 0.f : 1.f;
 
   // operand columns beyond the padded arrays are clamped (they feed accumulators that
-  // are never stored)
-  const float2* pa = g.A + ((long)bin * g.Kp + h) * g.Ip + min(r, g.Ip - 1);
-  const float2* pb = g.B + ((long)bin * g.Kp + h) * g.Jp + min(r, g.Jp - 1);
-  const long sa = 2L * g.Ip, sb = 2L * g.Jp;  // two k-rows
+  // are never stored).  An address is a scalar base (bin, k-rows) plus the lane's fixed
+  // 32-bit offset: no vector arithmetic per load.
+  const unsigned laneA = (unsigned)(h * g.Ip + min(r, g.Ip - 1)) * (unsigned)sizeof(float2);
+  const unsigned laneB = (unsigned)(h * g.Jp + min(r, g.Jp - 1)) * (unsigned)sizeof(float2);
+  const char* const binA = (const char*)(g.A + (long)bin * g.Kp * g.Ip);
+  const char* const binB = (const char*)(g.B + (long)bin * g.Kp * g.Jp);
+  const long sa = 2L * g.Ip * sizeof(float2), sb = 2L * g.Jp * sizeof(float2);  // two k-rows
 
   floatx16 k1, k2, k3;
 #pragma unroll
   for (int v = 0; v < 16; ++v) k1[v] = k2[v] = k3[v] = 0.f;
 
   auto fetch = [&](GemmSlice& s, int sl) __attribute__((always_inline)) {
-    const float2* qa = pa + (long)sl * (GK2 / 2) * sa;
-    const float2* qb = pb + (long)sl * (GK2 / 2) * sb;
 #pragma unroll
     for (int u = 0; u < GK2 / 2; ++u) {
-      s.a[u] = qa[u * sa];
-      s.b[u] = qb[u * sb];
+      const long k2rows = (long)sl * (GK2 / 2) + u;
+      const PlainPair va = *(const GlobalPair*)(scalarBase(binA + k2rows * sa) + laneOffset(laneA));
+      const PlainPair vb = *(const GlobalPair*)(scalarBase(binB + k2rows * sb) + laneOffset(laneB));
+      s.a[u] = float2{va.x, va.y};
+      s.b[u] = float2{vb.x, vb.y};
     }
   };
   // a conj(b) = (k1 - k3) + i (k1 + k2) with k1 = (ar + ai) br, k2 = -ar (br + bi),
@@ -705,8 +771,7 @@ __global__ __launch_bounds__(kT, 4) void binGemmRegsSplitK(GemmArgs g) {
       const int i = 8 * (v / 4) + 4 * h + v % 4;
       if (i < g.I)
         Cb[(long)i * g.Jp + r] =
-            pairs ? float2{k1[v] * g.invNorm, -k3[v] * g.invNorm}
-                  : float2{(k1[v] - k3[v]) * g.invNorm, (k1[v] + k2[v]) * g.invNorm};
+            pairs ? float2{k1[v], -k3[v]} : float2{k1[v] - k3[v], k1[v] + k2[v]};
     }
   }
 }
@@ -725,7 +790,7 @@ struct GemmSliceWide {
 
 __global__ __launch_bounds__(kT, 3) void binGemmRegsWide(GemmArgs g) {
   const int t = threadIdx.x;
-  const int lane = t % 64, w = t / 64;
+  const int lane = t % 64, w = __builtin_amdgcn_readfirstlane(t / 64);
   const int r = lane % 32, h = lane / 32;
   // g.IT: 32-row blocks, g.JT: workgroups (4 x 64 columns) along j
   const int total = g.bins * g.IT * g.JT;
@@ -741,9 +806,12 @@ __global__ __launch_bounds__(kT, 3) void binGemmRegsWide(GemmArgs g) {
 
   // operand columns beyond the padded arrays are clamped (they feed accumulators that
   // are never stored); Jp is even and rows of B and C start on 16-byte boundaries
-  const float2* pa = g.A + ((long)bin * g.Kp + h) * g.Ip + min(i0 + r, g.Ip - 1);
-  const float2* pb = g.B + ((long)bin * g.Kp + h) * g.Jp + min(j0 + 2 * r, g.Jp - 2);
-  const long sa = 2L * g.Ip, sb = 2L * g.Jp;  // two k-rows
+  // (an address: a scalar base - bin, k-rows, column block - plus the lane's fixed offset)
+  const unsigned laneA = (unsigned)(h * g.Ip + min(i0 + r, g.Ip - 1)) * (unsigned)sizeof(float2);
+  const unsigned laneB = (unsigned)(h * g.Jp + min(2 * r, g.Jp - 2 - j0)) * (unsigned)sizeof(float2);
+  const char* const binA = (const char*)(g.A + (long)bin * g.Kp * g.Ip);
+  const char* const binB = (const char*)(g.B + (long)bin * g.Kp * g.Jp + j0);
+  const long sa = 2L * g.Ip * sizeof(float2), sb = 2L * g.Jp * sizeof(float2);  // two k-rows
 
   floatx16 k1[2], k2[2], k3[2];
 #pragma unroll
@@ -752,12 +820,13 @@ __global__ __launch_bounds__(kT, 3) void binGemmRegsWide(GemmArgs g) {
     for (int v = 0; v < 16; ++v) k1[q][v] = k2[q][v] = k3[q][v] = 0.f;
 
   auto fetch = [&](GemmSliceWide& s, int sl) __attribute__((always_inline)) {
-    const float2* qa = pa + (long)sl * (GK2 / 2) * sa;
-    const float2* qb = pb + (long)sl * (GK2 / 2) * sb;
 #pragma unroll
     for (int u = 0; u < GK2 / 2; ++u) {
-      s.a[u] = qa[u * sa];
-      s.b[u] = *reinterpret_cast<const float4*>(qb + u * sb);
+      const long k2rows = (long)sl * (GK2 / 2) + u;
+      const PlainPair va = *(const GlobalPair*)(scalarBase(binA + k2rows * sa) + laneOffset(laneA));
+      const PlainQuad vb = *(const GlobalQuad*)(scalarBase(binB + k2rows * sb) + laneOffset(laneB));
+      s.a[u] = float2{va.x, va.y};
+      s.b[u] = float4{vb.x, vb.y, vb.z, vb.w};
     }
   };
   // a conj(b) = (k1 - k3) + i (k1 + k2) with k1 = (ar + ai) br, k2 = -ar (br + bi),
@@ -791,11 +860,10 @@ __global__ __launch_bounds__(kT, 3) void binGemmRegsWide(GemmArgs g) {
       if (i < g.I) {
         float4 o;
         if (pairs)
-          o = float4{k1[0][v] * g.invNorm, -k3[0][v] * g.invNorm, k1[1][v] * g.invNorm,
-                     -k3[1][v] * g.invNorm};
+          o = float4{k1[0][v], -k3[0][v], k1[1][v], -k3[1][v]};
         else
-          o = float4{(k1[0][v] - k3[0][v]) * g.invNorm, (k1[0][v] + k2[0][v]) * g.invNorm,
-                     (k1[1][v] - k3[1][v]) * g.invNorm, (k1[1][v] + k2[1][v]) * g.invNorm};
+          o = float4{k1[0][v] - k3[0][v], k1[0][v] + k2[0][v], k1[1][v] - k3[1][v],
+                     k1[1][v] + k2[1][v]};
         *reinterpret_cast<float4*>(Cb + (long)i * g.Jp + j) = o;
       }
     }
@@ -958,7 +1026,6 @@ int runPipeline(PlaneSet x, PlaneSet y, PlaneSet out, bool conjY, float scale, b
   g.Ip = Ip;
   g.Jp = Jp;
   g.Kp = Kp;
-  g.invNorm = 1.0f / (float)(N * N);
   const GemmPlan plan = planGemm(bins, I, Jp, Kp);
   g.IT = plan.IT;
   g.JT = plan.JT;
@@ -981,9 +1048,11 @@ int runPipeline(PlaneSet x, PlaneSet y, PlaneSet out, bool conjY, float scale, b
   // windows whose rows start on 8-byte boundaries with an even width: a lane stores its
   // two columns of a row as one 8-byte word
   const int po = movesAsPairs(out);
+  // the unnormalised transforms' 1 / N^2 (a power of two: exact) rides on the caller's factor
+  const float invNorm = 1.0f / (float)(N * N);
   auto launchInverse = [&](auto acc, auto groups, auto pairs) {
     inverseBinMajor<N, decltype(acc)::value, decltype(groups)::value, decltype(pairs)::value>
-        <<<igrid, dim3(kTF), 0, s>>>(SC, I, Jp, out, scale, g.splits, g.splitStride);
+        <<<igrid, dim3(kTF), 0, s>>>(SC, I, Jp, out, scale * invNorm, g.splits, g.splitStride);
   };
   auto withPairs = [&](auto acc, auto groups) {
     if (po == 2)

@@ -492,6 +492,20 @@ struct DirectA0 {
 
 __device__ __forceinline__ int directSlot(int row16, int pair) { return 4 * row16 + (pair ^ (row16 / 4)); }
 
+// A wave-uniform address pinned in scalar registers, and a lane's 32-bit offset kept
+// apart from it up to the memory instruction: the empty statements keep the compiler
+// from folding the two into a 64-bit vector addition per access, so that "scalar base +
+// lane offset" reaches the instruction as its two operands.
+template <class T>
+__device__ __forceinline__ T* scalarBase(T* p) {
+  asm volatile("" : "+s"(p));
+  return p;
+}
+__device__ __forceinline__ unsigned laneOffset(unsigned& o) {
+  asm volatile("" : "+v"(o));  // in place: the register is the same before and after, no copy
+  return o;
+}
+
 __device__ __forceinline__ void loadToLds(const float* src, float4* ldsWaveBase) {
   __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
                                    (__attribute__((address_space(3))) void*)ldsWaveBase, 16, 0, 0);
@@ -518,27 +532,33 @@ __device__ __forceinline__ void transposeMMDirectBody(const MMArgs& a, int logic
   const int j0 = (rem % tilesJ) * DTJ;
   const int i0 = (rem / tilesJ) * DTI;
 
-  // loader role: wave w brings k-row w of every slice
-  const float* srcA[DTI / 16];
-  const float* srcB[DTJ / 16];
+  // loader role: wave w brings k-row w of every slice.  An address is a scalar base
+  // (tile and k) plus a lane's byte offset within the tile, which never changes;
+  // tiles whose rows lie too far apart for 32 bits are left to the other kernel by
+  // the launcher.
+  unsigned laneA[DTI / 16], laneB[DTJ / 16];
   {
     const int r = lane / 4, pair = (lane % 4) ^ (r / 4);
-    const long xoff = 2L * min(x0 + 2 * pair, a.XY - 2);
+    const long xoff = 2L * (min(x0 + 2 * pair, a.XY - 2) - x0);
 #pragma unroll
     for (int g = 0; g < DTI / 16; ++g)
-      srcA[g] = a.A + (long)min(i0 + 16 * g + r, a.I - 1) * a.aRow + xoff;
+      laneA[g] = (unsigned)(((long)(min(i0 + 16 * g + r, a.I - 1) - i0) * a.aRow + xoff) * (long)sizeof(float));
 #pragma unroll
     for (int g = 0; g < DTJ / 16; ++g)
-      srcB[g] = a.B + (long)min(j0 + 16 * g + r, a.J - 1) * a.bCol + xoff;
+      laneB[g] = (unsigned)(((long)(min(j0 + 16 * g + r, a.J - 1) - j0) * a.bCol + xoff) * (long)sizeof(float));
   }
+  const char* const tileA = (const char*)(a.A + (long)i0 * a.aRow + 2L * x0);
+  const char* const tileB = (const char*)(a.B + (long)j0 * a.bCol + 2L * x0);
   const int slices = ceilDiv(a.K, KC);
   auto issue = [&](auto& stA, auto& stB, int sl) __attribute__((always_inline)) {
     const int k = min(sl * KC + w, a.K - 1);  // past the end: the last k again, zeroed before use
-    const long offA = (long)k * a.aK, offB = (long)k * a.bK;
+    const long offA = (long)k * a.aK * (long)sizeof(float), offB = (long)k * a.bK * (long)sizeof(float);
 #pragma unroll
-    for (int g = 0; g < DTI / 16; ++g) loadToLds(srcA[g] + offA, &stA.v[w][g][0]);
+    for (int g = 0; g < DTI / 16; ++g)
+      loadToLds((const float*)(scalarBase(tileA + offA) + laneOffset(laneA[g])), &stA.v[w][g][0]);
 #pragma unroll
-    for (int g = 0; g < DTJ / 16; ++g) loadToLds(srcB[g] + offB, &stB.v[w][g][0]);
+    for (int g = 0; g < DTJ / 16; ++g)
+      loadToLds((const float*)(scalarBase(tileB + offB) + laneOffset(laneB[g])), &stB.v[w][g][0]);
   };
 
   // reader role: the lane supplies row/col lane%32 (+32 for the second sub-tile of A)
@@ -548,8 +568,9 @@ __device__ __forceinline__ void transposeMMDirectBody(const MMArgs& a, int logic
   const int readA = (kpar * (DTI / 16) + rg) * 64 + slot, readB = (kpar * (DTJ / 16) + rg) * 64 + slot;
   const float sA = a.aSign, sB = a.bSign;
 
-  // [bin of the pair][sub-tile of A]; a b = (k1 - k3) + i (k1 + k2) for
-  //   k1 = (ar + sA ai) br,  k2 = ar (sB bi - br),  k3 = ai (sA br + sA sB bi)
+  // [bin of the pair][sub-tile of A]; a b = (k1 - sA k3) + i (k1 + k2) for
+  //   k1 = (ar + sA ai) br,  k2 = ar (sB bi - br),  k3 = ai (br + sB bi)
+  // (sA = +-1 is applied to k3 once, on the way out, not to every operand sum)
   floatx16 k1[2][SI], k2[2][SI], k3[2][SI];
 #pragma unroll
   for (int h = 0; h < 2; ++h)
@@ -602,7 +623,7 @@ __device__ __forceinline__ void transposeMMDirectBody(const MMArgs& a, int logic
 #pragma unroll
       for (int h = 0; h < 2; ++h) {
         const float bd = __builtin_fmaf(sB, bi[h], -br[h]);
-        const float bs = sA * __builtin_fmaf(sB, bi[h], br[h]);
+        const float bs = __builtin_fmaf(sB, bi[h], br[h]);
 #pragma unroll
         for (int si = 0; si < SI; ++si) {
           const float ar = h ? av[s2][si].z : av[s2][si].x, ai = h ? av[s2][si].w : av[s2][si].y;
@@ -653,14 +674,46 @@ __device__ __forceinline__ void transposeMMDirectBody(const MMArgs& a, int logic
           const float v1 = k1[h][si][4 * c + rr], v2 = k2[h][si][4 * c + rr],
                       v3 = k3[h][si][4 * c + rr];
           st[(((DCR == 8 ? 4 * hh : 0) + rr) * DTJ + col) * CSTR + 2 * w + h] =
-              float2{v1 - v3, v1 + v2};
+              float2{__builtin_fmaf(-sA, v3, v1), v1 + v2};
         }
     }
   };
   const int q = t % 4;
+  // A tile that lies inside C whole (all but the last row, column or bin group of
+  // tiles): an element's address is a scalar base per chunk and pass plus the lane's
+  // fixed 32-bit offset, no tests and no 64-bit vector arithmetic per store.
+  constexpr int ROWS_PER_PASS = DTHREADS / 4 / DTJ;
+  const bool whole = i0 + DTI <= a.I && j0 + DTJ <= a.J && x0 + XB <= a.XY &&
+                     (ROWS_PER_PASS * a.cRow + DTJ * a.cCol + 2 * XB) * (long)sizeof(float) < (1L << 31) &&
+                     a.cRow >= 0 && a.cCol >= 0;
+  unsigned laneC =
+      (unsigned)((t / 4 / DTJ) * a.cRow + (t / 4 % DTJ) * a.cCol + 4 * q) * (unsigned)sizeof(float);
+  char* const tileC = (char*)(a.C + (long)i0 * a.cRow + (long)j0 * a.cCol + 2L * x0);
   auto store = [&](auto nn) __attribute__((always_inline)) {
     constexpr int n = decltype(nn)::value, si = n / (4 * PER8), c = n / PER8 % 4, half = n % PER8;
     const float2* st = stg[n % 2];
+    if (whole) {
+      auto put = [&](auto accumulating) __attribute__((always_inline)) {
+#pragma unroll
+        for (int pass = 0; pass < DCR * DTJ * 4 / DTHREADS; ++pass) {
+          const int e = t / 4 + (DTHREADS / 4) * pass;
+          const float2 c0 = st[e * CSTR + 2 * q], c1 = st[e * CSTR + 2 * q + 1];
+          typedef float __attribute__((ext_vector_type(4))) Quad;  // (float4's assignment takes a generic `this`)
+          auto* dst = (__attribute__((address_space(1))) Quad*)(
+              scalarBase(tileC + (32 * si + 8 * c + 4 * half + ROWS_PER_PASS * pass) * a.cRow *
+                                     (long)sizeof(float)) +
+              laneOffset(laneC));
+          Quad acc{c0.x, c0.y, c1.x, c1.y};
+          if constexpr (decltype(accumulating)::value) acc += *dst;
+          *dst = acc * a.invNorm;
+        }
+      };
+      if (a.accumulate)
+        put(std::true_type{});
+      else
+        put(std::false_type{});
+      return;
+    }
 #pragma unroll
     for (int pass = 0; pass < DCR * DTJ * 4 / DTHREADS; ++pass) {
       const int e = t / 4 + (DTHREADS / 4) * pass;
@@ -776,7 +829,9 @@ int launchTransposeMM(const float* A, long a0, long a1, const float* B, long b0,
   const MMArgs m = makeArgs(A, a0, a1, B, b0, b1, C, c0, c1, I, J, K, XY, conjA, conjB, accumulate,
                             invNorm, ceilDiv(XY, XB));
   const bool vec4 = movesAsFloat4(A, a0, a1, B, b0, b1, XY);
-  if (vec4 && storesAsFloat4(C, c0, c1)) {
+  // (the fast path keeps a lane's offset within its tile, up to 63 rows, in 32 bits)
+  const bool rowsNear = m.aRow >= 0 && m.aRow < (1L << 24) && m.bCol >= 0 && m.bCol < (1L << 24);
+  if (vec4 && rowsNear && storesAsFloat4(C, c0, c1)) {
     // Equal work items are dealt to the CUs in whole numbers: the launch lasts as
     // long as the fullest CU.  32-row tiles re-read B twice as often and pay more per
     // matrix instruction, so they are taken only where they even the load out
