@@ -410,8 +410,8 @@ struct GemmArgs {
 };
 
 // The k-slices go from HBM straight into LDS (global_load_lds, 16 bytes per lane,
-// no staging registers or LDS store instructions) through a ring of four stages:
-// slice s+3 is requested before slice s is multiplied, one barrier per slice.  A
+// no staging registers or LDS store instructions) through a ring of three stages:
+// slice s+2 is requested before slice s is multiplied, one barrier per slice.  A
 // wave instruction moves 1 KiB: one k-row of 128 complex or two k-rows of 64
 // complex; LDS has exactly the HBM layout.  Requires Kp % 8 == 0 with the padding
 // rows zeroed; rows / columns beyond Ip / Jp are clamped (they only feed
@@ -459,15 +459,15 @@ struct GemmStage {
 // TI = 64 (few rows, or too few 128-row tiles to balance the chip): wave w owns rows
 // 32 (w % 2).. and columns 32 (w / 2)..
 template <int TI>
-__global__ __launch_bounds__(kT, TI == 128 ? 3 : 4) void binGemmDirect(GemmArgs g) {
+__global__ __launch_bounds__(kT, TI == 128 ? 4 : 6) void binGemmDirect(GemmArgs g) {
   static_assert(TI == 128 || TI == 64, "tile rows");
   constexpr int NQ = TI == 128 ? 2 : 1;
   constexpr int LOADS = TI == 128 ? 3 : 2;  // global->LDS instructions per wave and slice
   using Stage = GemmStage<TI>;
-  // four separate variables, not one array: the compiler tracks pending
+  // three separate variables, not one array: the compiler tracks pending
   // global->LDS loads per LDS variable, so reading one stage does not wait for the
   // loads still in flight into the other three
-  __shared__ __align__(16) Stage stage0, stage1, stage2, stage3;
+  __shared__ __align__(16) Stage stage0, stage1, stage2;
   const int t = threadIdx.x;
   const int lane = t % 64;
   // the wave's number in a scalar register: everything below that depends only on it
@@ -501,6 +501,10 @@ __global__ __launch_bounds__(kT, TI == 128 ? 3 : 4) void binGemmDirect(GemmArgs 
   //   k1 = (ar + ai) br,  k2 = -ar (br + bi),  k3 = ai (br - bi).
   // The sums cost three VALU adds per operand pair; the matrix pipeline, which
   // bounds this kernel, does a quarter less work.
+  // (Cleared by 48 moves per sub-tile.  Giving the first slice's products a constant
+  // zero addend instead takes that slice out of the loop, and there the compiler waits
+  // for every load in flight before the first LDS read: 101 -> 107 us on a
+  // 128 x 64 x 27 x 27 * 192 x 64 x 5 x 5 forward pass.)
   floatx16 k1[NQ], k2[NQ], k3[NQ];
 #pragma unroll
   for (int q = 0; q < NQ; ++q)
@@ -528,20 +532,23 @@ __global__ __launch_bounds__(kT, TI == 128 ? 3 : 4) void binGemmDirect(GemmArgs 
     loadToLds((const float2*)(scalarBase(waveB + sl * sliceB) + laneOffset(laneB)), &st.B[2 * w][0]);
   };
 
-  // One slice: wait for it, let everybody see it, request the slice three ahead into
+  // One slice: wait for it, let everybody see it, request the slice two ahead into
   // the stage that was multiplied last time round, multiply.  Every step issues
   // exactly LOADS loads (past the end it re-requests the last slice into a stage
-  // nobody reads), so "all but the newest 2 LOADS have landed" always means "slice sl
+  // nobody reads), so "all but the newest LOADS have landed" always means "slice sl
   // has landed" and the compiler can count the loads in flight at every LDS read.
-  // (Three slices in flight instead of two: the weight gradient of configs[3], sixteen
-  // slices per workgroup, 104.8 -> 102.6 us; the forward pass, eight slices, unchanged.)
+  // (Three stages of 8 KB let six workgroups of the 64-row kernel share a CU, 74
+  // registers per lane allowing it; a fourth stage with five workgroups measured 0.6 /
+  // 0.8 / 2.5 us slower on the three passes of a 128 x 64 x 27 x 27 * 192 x 64 x 5 x 5
+  // layer - while the kernel needed 89 registers and five workgroups were the most
+  // either way, the fourth stage was the faster form by 2 us on the weight gradient.)
   auto step = [&](Stage& cur, Stage& refill, int sl) __attribute__((always_inline)) {
-    __builtin_amdgcn_s_waitcnt(0x0F70 | (2 * LOADS));  // vmcnt(2 LOADS): all but the newest two slices
+    __builtin_amdgcn_s_waitcnt(0x0F70 | LOADS);  // vmcnt(LOADS): all but the newest slice
     // ... and so have everybody else's, and slice sl-1 is consumed.  A bare barrier:
     // the fences of __syncthreads() would wait for every load in flight, and no wave
     // stores to LDS with anything but these loads.
     __builtin_amdgcn_s_barrier();
-    issue(refill, min(sl + 3, slices - 1));
+    issue(refill, min(sl + 2, slices - 1));
     float2 av[GK2 / 2], bv[GK2 / 2][NQ];
 #pragma unroll
     for (int s2 = 0; s2 < GK2 / 2; ++s2) {
@@ -566,18 +573,15 @@ __global__ __launch_bounds__(kT, TI == 128 ? 3 : 4) void binGemmDirect(GemmArgs 
 
   issue(stage0, 0);
   issue(stage1, min(1, slices - 1));
-  issue(stage2, min(2, slices - 1));
   int sl = 0;
-  for (; sl + 4 <= slices; sl += 4) {
-    step(stage0, stage3, sl);
+  for (; sl + 3 <= slices; sl += 3) {
+    step(stage0, stage2, sl);
     step(stage1, stage0, sl + 1);
     step(stage2, stage1, sl + 2);
-    step(stage3, stage2, sl + 3);
   }
   if (sl < slices) {
-    step(stage0, stage3, sl);
+    step(stage0, stage2, sl);
     if (sl + 1 < slices) step(stage1, stage0, sl + 1);
-    if (sl + 2 < slices) step(stage2, stage1, sl + 2);
   }
   __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): nothing may land in LDS after this wave is gone
 
