@@ -104,11 +104,16 @@ struct ConvCfg {
   static_assert(BN * FQ * NBT == 64, "64 complex accumulators per lane");
 };
 
-// a (x) w for the pass: a * conj(w) or a * w
+// acc += a (x) w for the pass: a * conj(w) or a * w.  Four chained multiply-adds: formed
+// as a product that is then added, it is six instructions (multiply, multiply-add and
+// add per component - the compiler may not reassociate the sum), and this kernel is
+// bound by the vector instructions it issues.
 template <bool CONJ>
-__device__ __forceinline__ c32 prod(c32 a, c32 w) {
-  return CONJ ? c32{a.x * w.x + a.y * w.y, a.y * w.x - a.x * w.y}
-              : c32{a.x * w.x - a.y * w.y, a.x * w.y + a.y * w.x};
+__device__ __forceinline__ void accumulate(c32& acc, c32 a, c32 w) {
+  acc.x = __builtin_fmaf(a.x, w.x, acc.x);
+  acc.x = __builtin_fmaf(CONJ ? a.y : -a.y, w.y, acc.x);
+  acc.y = __builtin_fmaf(a.y, w.x, acc.y);
+  acc.y = __builtin_fmaf(CONJ ? -a.x : a.x, w.y, acc.y);
 }
 
 // split a packed row-0 value into its two real-row spectra
@@ -208,11 +213,7 @@ __global__ __launch_bounds__(kThreads) void iteratedConvKernel(ConvArgs a) {
           for (int i = 0; i < BN; ++i) {
             const c32 av = ldsu[i * PSZ + o];
 #pragma unroll
-            for (int q = 0; q < FQ; ++q) {
-              const c32 p = prod<CONJ>(av, wv[q]);
-              acc[i][q][nb].x += p.x;
-              acc[i][q][nb].y += p.y;
-            }
+            for (int q = 0; q < FQ; ++q) accumulate<CONJ>(acc[i][q][nb], av, wv[q]);
           }
         } else {
           // Row 0.  v = this lane's real-row spectrum value of a plane: the row-0 or
@@ -245,13 +246,11 @@ __global__ __launch_bounds__(kThreads) void iteratedConvKernel(ConvArgs a) {
             const float a1y = pair ? 0.0f : av.y, a2x = pair ? 0.0f : av.x;
 #pragma unroll
             for (int q = 0; q < FQ; ++q) {
-              if (CONJ) {
-                acc[i][q][nb].x += av.x * wv[q].x + a1y * wv[q].y;
-                acc[i][q][nb].y += av.y * w2x[q] - a2x * wv[q].y;
-              } else {
-                acc[i][q][nb].x += av.x * wv[q].x - a1y * wv[q].y;
-                acc[i][q][nb].y += a2x * wv[q].y + av.y * w2x[q];
-              }
+              c32& to = acc[i][q][nb];
+              to.x = __builtin_fmaf(av.x, wv[q].x, to.x);
+              to.x = __builtin_fmaf(CONJ ? a1y : -a1y, wv[q].y, to.x);
+              to.y = __builtin_fmaf(av.y, w2x[q], to.y);
+              to.y = __builtin_fmaf(CONJ ? -a2x : a2x, wv[q].y, to.y);
             }
           }
         }
