@@ -146,6 +146,21 @@ __device__ __forceinline__ void loadColumnsWindowPerLane(const float* src, int s
     GlobalPtr2 pp = (GlobalPtr2)(src + xa - (long)padU * sy);
     const int sy2 = sy / 2;
     Pair r[N];
+    // ... and when every lane's window covers the whole transform (the inner tiles of a
+    // larger image), nothing is zeroed and nothing is tested row by row
+    const bool whole = padU == 0 && padL == 0 && h >= N && w >= N;
+    if (__builtin_amdgcn_ballot_w64(!whole) == 0) {
+      staticFor<N>([&](auto yy) {
+        constexpr int y = decltype(yy)::value;
+        r[y] = pp[(long)y * sy2];
+      });
+      staticFor<N / 2>([&](auto jj) {
+        constexpr int j = decltype(jj)::value;
+        z0[j] = c32{r[2 * j].x, r[2 * j + 1].x};
+        z1[j] = c32{r[2 * j].y, r[2 * j + 1].y};
+      });
+      return;
+    }
     staticFor<N>([&](auto yy) {
       constexpr int y = decltype(yy)::value;
       r[y] = Pair{0.0f, 0.0f};
