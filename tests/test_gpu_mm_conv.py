@@ -363,6 +363,36 @@ def test_conv_layer_random_shapes(oracle, seed):
     assert rel(gw.cpu().numpy(), 2.0 * oracle.corr2d_grad_weight(xh, gh, kH, kW)) < TOL_CONV, tag
 
 
+@pytest.mark.parametrize("seed", range(8))
+def test_conv_layer_random_shapes_many_planes(oracle, seed):
+    """All three passes on seeded random layers whose plane counts (33 .. 72 images and
+    output planes, 3 .. 40 input planes) put more than 32 rows on both sides of the
+    per-bin contraction: 64-row and 128-row tiles that lie inside the product whole next
+    to tiles that hang over its edges, reductions with and without a partial last slice."""
+    rng = np.random.default_rng(5000 + seed)
+    N = int(rng.choice([8, 16]))
+    H, W = int(rng.integers(N // 2, N + 1)), int(rng.integers(N // 2, N + 1))
+    kH, kW = int(rng.integers(1, 4)), int(rng.integers(1, 4))
+    Bn, Cin, Cout = int(rng.integers(33, 73)), int(rng.integers(3, 41)), int(rng.integers(33, 73))
+    d = dev()
+    x = synth.normal((Bn, Cin, H, W), seed=seed, device=d)
+    w = synth.normal((Cout, Cin, kH, kW), seed=seed + 100, std=0.1, device=d)
+    go = synth.normal((Bn, Cout, H - kH + 1, W - kW + 1), seed=seed + 200, device=d)
+    tag = (N, H, W, kH, kW, Bn, Cin, Cout)
+    xh, wh, gh = x.cpu().numpy(), w.cpu().numpy(), go.cpu().numpy()
+
+    out = torch.full_like(go, float("nan"))
+    assert F.conv_fprop(x, w, out, N, workspace(0, Bn, Cin, Cout, N)) == F.Success
+    gi = torch.full_like(x, float("nan"))
+    assert F.conv_bprop(go, w, gi, N, workspace(1, Bn, Cin, Cout, N)) == F.Success
+    gw = torch.full_like(w, float("nan"))
+    assert F.conv_accgrad(x, go, gw, N, workspace(2, Bn, Cin, Cout, N)) == F.Success
+    torch.cuda.synchronize()
+    assert rel(out.cpu().numpy(), oracle.corr2d_valid(xh, wh)) < TOL_CONV, tag
+    assert rel(gi.cpu().numpy(), oracle.corr2d_grad_input(gh, wh, H, W)) < TOL_CONV, tag
+    assert rel(gw.cpu().numpy(), oracle.corr2d_grad_weight(xh, gh, kH, kW)) < TOL_CONV, tag
+
+
 @pytest.mark.parametrize("Cin", [5, 8, 12, 24, 40])
 def test_conv_fprop_many_full_tiles(oracle, Cin):
     """512 x 512 outputs per bin in 8-point transforms: more 64 x 64 tiles of the contraction
