@@ -446,3 +446,26 @@ def test_mm_both_tile_shapes_of_the_aligned_path(oracle, I, J, K, shape):
         want = oracle.transpose_mm(A.reshape(A.shape[0], A.shape[1], xy, 2),
                                    B.reshape(B.shape[0], B.shape[1], xy, 2), conjA, conjB, 0.5)
         assert rel(got.reshape(I, J, xy, 2), want) < TOL_FFT
+
+
+@pytest.mark.parametrize("seed", range(10))
+def test_mm_random_aligned_shapes(oracle, seed):
+    """Seeded random draw over contiguous operands with an even bin count (the kernel that
+    copies slices straight into LDS): I and J from below one tile to several, so that tiles
+    inside C whole - stored from a scalar base without tests - meet tiles that hang over its
+    last rows, columns or bins; every role, with and without accumulation."""
+    rng = np.random.default_rng(6000 + seed)
+    I, J, K = int(rng.integers(20, 200)), int(rng.integers(20, 200)), int(rng.integers(1, 80))
+    shape = (int(rng.integers(1, 6)), 2 * int(rng.integers(1, 9)))
+    xy = shape[0] * shape[1]
+    conjA, conjB = ROLES[int(rng.integers(0, 3))]
+    acc = bool(rng.integers(0, 2))
+    A = synth.normal(((K, I) if conjA else (I, K)) + shape + (2,), seed=21 + seed).numpy()
+    B = synth.normal(((J, K) if conjB else (K, J)) + shape + (2,), seed=22 + seed).numpy()
+    C0 = synth.normal((I, J) + shape + (2,), seed=23 + seed).numpy()
+    rc, got = mm(A, B, conjA, conjB, 0.25, C0=C0 if acc else None)
+    assert rc == F.Success
+    want = oracle.transpose_mm(A.reshape(A.shape[0], A.shape[1], xy, 2),
+                               B.reshape(B.shape[0], B.shape[1], xy, 2), conjA, conjB, 0.25,
+                               C=C0.reshape(I, J, xy, 2) if acc else None)
+    assert rel(got.reshape(I, J, xy, 2), want) < TOL_FFT, (I, J, K, shape, conjA, conjB, acc)
