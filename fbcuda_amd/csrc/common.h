@@ -29,6 +29,25 @@ __host__ __device__ __forceinline__ bool inWindow(int y, int x, int padU, int pa
 
 __host__ __device__ inline int ceilDiv(int a, int b) { return (a + b - 1) / b; }
 
+// Stores of results that the launch itself never reads back carry the nontemporal
+// hint: the lines are not kept in L2 or in the 256 MiB last-level cache on their way to
+// HBM, so they do not push the operands still to be read out of it.  Measured on
+// batches larger than that cache: 32 x 32 R2C of 65536 planes 100.4 -> 85.9 us (5.5 ->
+// 6.4 TB/s), 16 x 16 98.6 -> 87.9 us, 8 x 8 105.0 -> 86.7 us; the same hint on the loads
+// costs 5 %.  Operands that stay in the cache from one launch to the next (the same
+// 132 MB over and over) lose 2-3 %.
+typedef float vfloat2 __attribute__((ext_vector_type(2)));
+typedef float vfloat4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ void streamStore(float4* p, float4 v) {
+  __builtin_nontemporal_store(vfloat4{v.x, v.y, v.z, v.w}, reinterpret_cast<vfloat4*>(p));
+}
+__device__ __forceinline__ void streamStore(float2* p, float2 v) {
+  __builtin_nontemporal_store(vfloat2{v.x, v.y}, reinterpret_cast<vfloat2*>(p));
+}
+__device__ __forceinline__ void streamStore(float* p, float v) {
+  __builtin_nontemporal_store(v, p);
+}
+
 inline bool aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
 
 // status of the launches just made; the error is consumed, so that one failed

@@ -345,7 +345,7 @@ __global__ __launch_bounds__(k1dThreads, 2) void fft1dMidForward(const float* __
   const int total = rows * RS;  // complex values of this workgroup
   float4* dst = reinterpret_cast<float4*>(cplx + (size_t)b0 * 2 * RS);
   const float4* l4 = reinterpret_cast<const float4*>(lds);
-  for (int q = t; q < total / 2; q += k1dThreads) dst[q] = l4[q];
+  for (int q = t; q < total / 2; q += k1dThreads) streamStore(dst + q, l4[q]);
   if ((total & 1) && t == 0)
     reinterpret_cast<float2*>(cplx + (size_t)b0 * 2 * RS)[total - 1] = lds[total - 1];
 }
@@ -539,7 +539,7 @@ __global__ __launch_bounds__(k1dThreads, 2) void fft1dMidInverse(const float* __
       o = float4{base[f] + sg * base[H + f], base[f + 1] + sg * base[H + f + 1],
                  base[f + 2] + sg * base[H + f + 2], base[f + 3] + sg * base[H + f + 3]};
     }
-    dst[q] = o;
+    streamStore(dst + q, o);
   }
 }
 

@@ -244,7 +244,7 @@ __global__ __launch_bounds__(LargeCfg<N>::THREADS) void fft2dLargeForward(RealVi
         o = float4{a0.x, a0.y, a1.x, a1.y};
       }
       if constexpr (FAST_CPLX) {
-        reinterpret_cast<float4*>(cplx.data + (size_t)b * cplx.sb)[q] = o;
+        streamStore(reinterpret_cast<float4*>(cplx.data + (size_t)b * cplx.sb) + q, o);
       } else {
         float* dst = cplx.data + (size_t)b * cplx.sb + (size_t)r * cplx.sr + (size_t)ky * cplx.sc;
         *reinterpret_cast<float2*>(dst) = float2{o.x, o.y};
@@ -343,7 +343,7 @@ __global__ __launch_bounds__(LargeCfg<N>::THREADS) void fft2dLargeInverse(CplxVi
         constexpr int i = decltype(ii)::value;
         const int q = t + THREADS * i;
         const int y = q / (N / 4), x4 = q % (N / 4);
-        dst[(size_t)y * rs4 + x4] = *reinterpret_cast<const float4*>(buf + y * RSF + 4 * x4);
+        streamStore(dst + (size_t)y * rs4 + x4, *reinterpret_cast<const float4*>(buf + y * RSF + 4 * x4));
       });
     } else {
       // a lane keeps its column and walks down the rows of the window
@@ -428,8 +428,8 @@ __global__ __launch_bounds__(LargeCfg<N>::THREADS) void fft2dLargeInverse(CplxVi
         const float4 e = *reinterpret_cast<const float4*>(buf + yy * RSF + f);
         const float4 w = *reinterpret_cast<const float4*>(buf + yy * RSF + H + f);
         const float sg = 4 * x4 < H ? 1.0f : -1.0f;
-        dst[(size_t)yy * rs4 + x4] =
-            float4{e.x + sg * w.x, e.y + sg * w.y, e.z + sg * w.z, e.w + sg * w.w};
+        streamStore(dst + (size_t)yy * rs4 + x4,
+                    float4{e.x + sg * w.x, e.y + sg * w.y, e.z + sg * w.z, e.w + sg * w.w});
       });
     } else {
       // a lane keeps its column and walks down the rows of the window

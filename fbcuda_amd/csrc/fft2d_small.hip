@@ -98,7 +98,7 @@ __global__ __launch_bounds__(64) void fft2dSmallForward(RealView real, CplxView 
         const int bo = b0 + pp0;
         if (FULL || bo < B) {
           if constexpr (FAST_CPLX) {
-            reinterpret_cast<float4*>(cplx.data + (size_t)bo * cplx.sb)[(r0 + g) * (N / 2) + xq] = v;
+            streamStore(reinterpret_cast<float4*>(cplx.data + (size_t)bo * cplx.sb) + (r0 + g) * (N / 2) + xq, v);
           } else {
             float* o = cplx.data + (size_t)bo * cplx.sb + (size_t)(r0 + g) * cplx.sr +
                        (size_t)(2 * xq) * cplx.sc;
@@ -131,7 +131,7 @@ __global__ __launch_bounds__(64) void fft2dSmallForward(RealView real, CplxView 
       const int bo = b0 + pp;
       if (FULL || bo < B) {
         if constexpr (FAST_CPLX) {
-          reinterpret_cast<float4*>(cplx.data + (size_t)bo * cplx.sb)[rem] = v;
+          streamStore(reinterpret_cast<float4*>(cplx.data + (size_t)bo * cplx.sb) + rem, v);
         } else {
           float* o = cplx.data + (size_t)bo * cplx.sb + (size_t)r * cplx.sr + (size_t)kx * cplx.sc;
           *reinterpret_cast<float2*>(o) = float2{v.x, v.y};
@@ -274,7 +274,7 @@ __global__ __launch_bounds__(64) void fft2dSmallInverse(CplxView cplx, RealView 
         staticFor<P * N * N / 4 / 64>([&](auto ii) {
           constexpr int i = decltype(ii)::value;
           const int q = lane + 64 * i;
-          if (q < valid) dst[q] = reinterpret_cast<const float4*>(stage)[q];
+          if (q < valid) streamStore(dst + q, reinterpret_cast<const float4*>(stage)[q]);
         });
         return;
       }
@@ -286,8 +286,8 @@ __global__ __launch_bounds__(64) void fft2dSmallInverse(CplxView cplx, RealView 
         staticFor<H>([&](auto jj) {
           constexpr int j = decltype(jj)::value;
           c32 a = z0[slot<H>(j)], c = z1[slot<H>(j)];
-          dst[(size_t)(2 * j) * rs2] = float2{a.x, c.x};
-          dst[(size_t)(2 * j + 1) * rs2] = float2{a.y, c.y};
+          streamStore(dst + (size_t)(2 * j) * rs2, float2{a.x, c.x});
+          streamStore(dst + (size_t)(2 * j + 1) * rs2, float2{a.y, c.y});
         });
       } else {
         storeColumnsWindow<N>(real.data + (size_t)b * real.sb, real.sy, real.sx, real.h, real.w,
@@ -313,18 +313,22 @@ __global__ __launch_bounds__(64) void fft2dSmallInverse(CplxView cplx, RealView 
 // Two groups per wave pay off only when the launch would otherwise take between
 // one and two rounds of resident waves: then the second round's load latency is
 // exposed, and folding it into the first round's waves (with their loads already
-// in flight) hides it.  Measured on 32 x 32 R2C: 26.9 -> 24.6 us at 16384 planes,
-// but 102 -> 113 us at 65536 planes, where other waves already cover the latency.
-// (Measured across the switch, 32 x 32 R2C, us per launch paired / unpaired: 9216 planes
-// 16.6 / 16.0, 10240 17.0 / 17.4, 12288 17.8 / 19.5, 14336 19.1 / 22.0, 16384 22.7 / 24.1;
-// a variant that keeps one full round of waves and gives only some of them a second
-// group was no better: 16.7, 17.0, 18.9, 20.3, 22.8.)
+// in flight) hides it.  Measured with operands that come from HBM (every launch on
+// another set of buffers, more than 1 GiB in all), 32 x 32 R2C, us per launch
+// paired / unpaired: 9216 planes 18.5 / 19.0, 10240 18.5 / 19.8, 12288 20.4 / 21.1,
+// 14336 23.7 / 25.0, but 16384 (exactly two groups for every resident wave, all of
+// them in step) 29.0 / 27.3; C2R 15.8 / 17.5, 16.6 / 18.4, 20.4 / 22.0, 24.0 / 25.0,
+// 28.2 / 27.6.  16 x 16 (30720 planes resident): 32768 planes 14.2 / 16.4, 36864
+// 16.7 / 17.6, 49152 21.8 / 21.9.  So waves pair up to 1.75 rounds; beyond that the
+// hardware's own replacement of finished workgroups spreads loads and stores better.
+// (On operands that stay in the last-level cache pairing is also ahead at 16384
+// planes, 21.7 against 22.5 us.)
 template <int N>
 bool pairGroups(int groups) {
   constexpr int ldsBytes = SmallCfg<N>::P * SmallCfg<N>::PS * (int)sizeof(c32);
   constexpr int wavesPerCU = (160 * 1024 / ldsBytes) < 32 ? (160 * 1024 / ldsBytes) : 32;
-  const int slots = computeUnits() * wavesPerCU;
-  return groups > slots && groups <= 2 * slots;
+  const long slots = (long)computeUnits() * wavesPerCU;
+  return groups > slots && 4L * groups <= 7 * slots;
 }
 
 bool fastReal(int N, const RealView& r, int padL, int padU) {

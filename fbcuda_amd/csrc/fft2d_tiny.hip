@@ -169,7 +169,7 @@ __device__ __forceinline__ void moveTiny(float* global, float* stage, int planes
       if constexpr (TO_LDS)
         *reinterpret_cast<float4*>(stage + (q / Q) * STRIDE + 4 * (q % Q)) = w;
       else
-        g4[q] = w;
+        streamStore(g4 + q, w);
     }
   });
 }
