@@ -2,18 +2,25 @@
 """Benchmark of the fbfft hot path on one MI355X.
 
 A step is one fbfft2D real-to-complex pass over the whole batch of
-BASELINE.json configs[1] (16384 planes of 32x32 fp32, N(0,1), seed 1), inputs
-resident in HBM.  Prints ONE JSON line:
+BASELINE.json configs[1] (16384 planes of 32x32 fp32, N(0,1)), inputs resident
+in HBM - and served from HBM: consecutive steps run on eight different sets of
+operand buffers (1.1 GB in all), because one set (132 MB) would sit in the 256 MiB
+last-level cache from one launch to the next.  Prints ONE JSON line:
 
   value / unit   algorithmic GB/s of the timed region (8448 bytes per plane:
                  4096 read + 4352 written), the metric BASELINE.json names
   roofline       the R2C kernel against the 8 TB/s HBM peak, duration from HIP
                  events recorded on the launch stream around the timed region
+  roofline_llc   the same launch on the same buffers every time (operands in
+                 the last-level cache), roofline_4x one launch over a 4x batch,
+                 copy_ceiling plain copies of the same bytes under the same
+                 rotation of buffers
   cpu_baseline   the CPU oracle (host transcription of the reference's
                  algorithm, OpenMP over planes) on the same workload, timed on
                  this machine's cores for a bounded number of passes
   extra          other measured configurations (C2R, other sizes, the FFT
-                 convolution of configs[3]) - informative, not the metric
+                 convolution of configs[3] with its own CPU baseline) -
+                 informative, not the metric
 """
 import argparse
 import ctypes
@@ -151,20 +158,97 @@ def cpu_baseline(x_host, N, budget_s=12.0):
             "single_thread_GBps": round(x_host.shape[0] * plane_bytes(N) / dt1 / 1e9, 3)}
 
 
-def profile_figure(name, key):
-    """An integer `key: value` line of a committed rocprofv3 summary under profiles/, or None."""
+def conv_cpu_baseline(budget_s=12.0):
+    """The reference's composition for configs[3] on the CPU oracle (kind "port"): fbfft2D of
+    the images and of the filters (FBFFT2D-inl.cuh:450-623), transposeMM with the filters
+    conjugate-transposed (MM-inl.cuh:515-814), fbifft2D with crop (FBIFFT2D-inl.cuh:567-742),
+    OpenMP over planes / (image, output plane) pairs.  Timed on a slice of the batch sized to
+    the budget; the filter transforms are charged once, the rest scales with the images."""
+    import numpy as np
+
+    from fbcuda_amd import synth
+    O, flags = native_oracle()
+    threads = O.num_threads()
+    cin, cout, N = 64, 192, 32
+    w = synth.normal((cout, cin, 5, 5), seed=31, std=0.02).numpy()
+
+    def run(x):
+        nb = x.shape[0]
+        t0 = time.perf_counter()
+        _, W = O.fbfft2d(w.reshape(-1, 5, 5), N)
+        t1 = time.perf_counter()
+        _, X = O.fbfft2d(x.reshape(-1, 27, 27), N)
+        C = O.transpose_mm(X.reshape(nb, cin, -1, 2), W.reshape(cout, cin, -1, 2), False, True,
+                           1.0 / (N * N))
+        _, out = O.fbifft2d(C.reshape(nb * cout, N // 2 + 1, N, 2), 23, 23)
+        t2 = time.perf_counter()
+        return t1 - t0, t2 - t1, out
+
+    x = synth.normal((128, cin, 27, 27), seed=30).numpy()
+    run(x[:1])                                    # warm
+    tw, tx, _ = run(x[:2])
+    nb = int(max(2, min(128, budget_s / max(tx / 2, 1e-4))))
+    tw, tx, out = run(x[:nb])
+    reps = 1
+    if nb == 128:   # the whole layer fits the budget several times over: average a few passes
+        reps = int(max(1, min(500, budget_s / max(tw + tx, 1e-3))))
+        acc = [run(x)[:2] for _ in range(reps)]
+        tw, tx = sum(a[0] for a in acc) / reps, sum(a[1] for a in acc) / reps
+    # sanity: one output pixel against its definition
+    ref = float(np.sum(x[0].astype(np.float64) [:, 3:8, 4:9] * w[5].astype(np.float64)))
+    got = float(out.reshape(nb, cout, 23, 23)[0, 5, 3, 4])
+    ms = (tw + tx * 128.0 / nb) * 1e3
+    return {"value": round(ms, 1), "unit": "ms/iter", "cores": threads, "kind": "port",
+            "sample": "%d pass(es) over %d of the 128 images of configs[3] with all 192x64 filters "
+                      "(%.2f s for the image-dependent part, %.3f s for the filter transforms per "
+                      "pass), scaled to 128 images" % (reps, nb, tx, tw),
+            "flags": flags, "check_abs_err": abs(got - ref)}
+
+
+CSRC = os.path.join(ROOT, "fbcuda_amd", "csrc")
+# the kernel sources each committed counter summary was measured on
+PROFILE_SOURCES = {
+    "fft2dSmallForward32_configs1.md": ("fft2d_small.hip", "fft2d_core.h", "fft_regs.h", "common.h"),
+    "conv_pipeline_configs3.md": ("conv_pipeline.hip", "fft2d_core.h", "fft_regs.h", "common.h"),
+    "conv_pipeline_configs4.md": ("conv_pipeline.hip", "fft2d_core.h", "fft_regs.h", "common.h"),
+}
+
+
+def source_sha16(files):
+    """First 16 hex digits of the SHA-256 over the named kernel sources, in order."""
+    import hashlib
+    h = hashlib.sha256()
+    for f in files:
+        with open(os.path.join(CSRC, f), "rb") as fh:
+            h.update(fh.read())
+    return h.hexdigest()[:16]
+
+
+def profile_traffic(name, key):
+    """(HBM bytes, where the figure comes from) read from a committed rocprofv3 counter
+    summary under profiles/.  The summary records the hash of the kernel sources it was
+    measured on (`kernel_source_sha16: ...`); when the sources have changed since, the
+    figure is withheld: (None, reason)."""
+    value = recorded = None
     try:
         for line in open(os.path.join(ROOT, "profiles", name)):
             if line.startswith(key + ":"):
-                return int(line.split(":")[1])
-    except (OSError, ValueError):
-        pass
-    return None
-
-
-def measured_traffic():
-    """HBM bytes per R2C launch from the committed rocprofv3 counter summary, or None."""
-    return profile_figure("fft2dSmallForward32_configs1.md", "traffic_bytes_per_launch")
+                value = int(line.split(":")[1])
+            elif line.startswith("kernel_source_sha16:"):
+                recorded = line.split(":")[1].split()[0]
+    except (OSError, ValueError, IndexError):
+        return None, "profiles/%s unreadable" % name
+    try:
+        current = source_sha16(PROFILE_SOURCES[name])
+    except OSError:
+        current = None
+    if value is None:
+        return None, "profiles/%s holds no %s" % (name, key)
+    if recorded is None or recorded != current:
+        return None, "profiles/%s was measured on other kernel sources (%s, now %s)" % (
+            name, recorded, current)
+    return value, "profiles/%s, rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on sources %s" % (
+        name, recorded)
 
 
 MFMA_FP32_PEAK = 157.3e12
@@ -198,12 +282,13 @@ def conv_extras(F, synth, torch, dev, extra):
     # the second half of the metric against its roofline: the whole iteration (forward
     # transforms, contraction, inverse transform) is charged to the contraction's matrix
     # work, 8 flop per complex multiply-add; frac_issued counts the 6 flop the kernels issue
+    tr3, tr3_src = profile_traffic("conv_pipeline_configs3.md", "traffic_bytes_per_iteration")
     extra["fft_conv_roofline"] = {
         "bound": "mfma", "achieved": round(CONV3_FLOP / t / 1e12, 2), "peak": MFMA_FP32_PEAK / 1e12,
         "unit": "TFLOP/s", "frac": round(CONV3_FLOP / t / MFMA_FP32_PEAK, 4),
         "frac_issued": round(CONV3_FLOP_ISSUED / t / MFMA_FP32_PEAK, 4),
         "floor_us": round(CONV3_FLOP / MFMA_FP32_PEAK * 1e6, 1), "iter_us": round(t * 1e6, 1),
-        "traffic": profile_figure("conv_pipeline_configs3.md", "traffic_bytes_per_iteration"),
+        "traffic": tr3, "traffic_source": tr3_src,
         "algorithmic_bytes": 77119488,
         "workload": "configs[3]: 128x64x27x27 * 192x64x5x5 -> 128x192x23x23, 32-point FFTs"}
     # the same pass with the transform size left to the library (fftSize 0): configs[3]
@@ -325,10 +410,11 @@ def conv_extras(F, synth, torch, dev, extra):
     extra["conv_layer_configs4_ms_per_iter_min"] = round(low * 1e3, 4)
     extra["conv_layer_configs4_direct_equiv_TFLOPs"] = round(163.3e9 / t / 1e12, 1)
     # 260.5 MB of algorithmic traffic (input + filters + output) against the HBM peak
+    tr4, tr4_src = profile_traffic("conv_pipeline_configs4.md", "traffic_bytes_per_iteration")
     extra["conv_layer_configs4_roofline"] = {
         "bound": "hbm", "achieved": round(260.5e6 / t / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
         "frac": round(260.5e6 / t / 1e9 / HBM_PEAK_GBS, 4), "algorithmic_bytes": 260500000,
-        "traffic": profile_figure("conv_pipeline_configs4.md", "traffic_bytes_per_iteration"),
+        "traffic": tr4, "traffic_source": tr4_src,
         "workload": "configs[4]: 16x32x256x256 * 32x32x9x9 -> 16x32x248x248, 32-point windows"}
     # the layer's other two passes on the same tiled image
     gi4, gw4 = torch.empty_like(x4), torch.empty_like(w4)
@@ -377,6 +463,23 @@ def run_only(name, steps, warmup, F, synth, torch, dev):
         fwd()
         fn = fwd if name.startswith("r2c") else prepared("fbfft_c2r_2d", F, spec, x, 0, 0)
         _, t = timed(fn, steps, warmup, torch)
+        return {"only": name, "us": round(t * 1e6, 2), "GBps": round(b * plane_bytes(n) / t / 1e9, 1)}
+    if name in ("r2c32hbm", "c2r32hbm"):
+        # configs[1] with operands served from HBM: eight sets of buffers in turn
+        n, b, sets = 32, 16384, 8
+        xs = [synth.normal((b, n, n), seed=1 + i, device=dev) for i in range(sets)]
+        ss = [torch.empty((b, n // 2 + 1, n, 2), device=dev) for _ in range(sets)]
+        fw = [prepared("fbfft_r2c_2d", F, xs[i], ss[i], 0, 0) for i in range(sets)]
+        for f in fw:
+            f()
+        cs = fw if name == "r2c32hbm" else [prepared("fbfft_c2r_2d", F, ss[i], xs[i], 0, 0)
+                                            for i in range(sets)]
+        turn = [0]
+
+        def step():
+            cs[turn[0] % sets]()
+            turn[0] += 1
+        _, t = timed(step, steps, warmup, torch)
         return {"only": name, "us": round(t * 1e6, 2), "GBps": round(b * plane_bytes(n) / t / 1e9, 1)}
     if name in ("r2c1d", "c2r1d"):
         n, b = 256, 1 << 18
@@ -466,15 +569,12 @@ def run_only(name, steps, warmup, F, synth, torch, dev):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    # defaults: 3000 launches of 23 us.  Launched over and over on the same 132 MB the
-    # kernel keeps getting faster for about a thousand launches (24 -> 22 us) while the
-    # last-level cache settles; the default warm-up runs past that.
-    ap.add_argument("--steps", type=int, default=2000)
-    ap.add_argument("--warmup", type=int, default=1000)
+    ap.add_argument("--steps", type=int, default=800)
+    ap.add_argument("--warmup", type=int, default=200)
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the informative extra configs")
     ap.add_argument("--only", default=None,
-                    choices=["r2c32", "c2r32", "r2c64", "c2r64", "r2c128", "c2r128", "mm", "conv",
+                    choices=["r2c32hbm", "c2r32hbm", "r2c32", "c2r32", "r2c64", "c2r64", "r2c128", "c2r128", "mm", "conv",
                              "conv_bprop", "conv_accgrad", "iterconv", "iter4", "iter4ws", "conv4",
                              "conv4_bprop", "conv4_accgrad", "r2c1d", "c2r1d"],
                     help="run just this workload --steps times (for rocprofv3) and print its timing")
@@ -510,16 +610,26 @@ def main():
         print(json.dumps(run_only(args.only, args.steps, args.warmup, F, synth, torch, dev)))
         return
 
-    N, B = 32, 16384
-    x = synth.normal((B, N, N), seed=1, device=dev)
-    spec = torch.empty((B, N // 2 + 1, N, 2), device=dev)
-    back = torch.empty_like(x)
-    fwd = prepared("fbfft_r2c_2d", F, x, spec, 0, 0)
-    inv = prepared("fbfft_c2r_2d", F, spec, back, 0, 0)
-
-    step_s, launch_s = timed(fwd, args.steps, args.warmup, torch)
-    launch_mid, launch_min = spread(fwd, args.steps, torch)
+    N, B, SETS = 32, 16384, 8
     nbytes = B * plane_bytes(N)
+    # Eight sets of operands (8 x 132 MB): a step runs on the set after the previous step's,
+    # so no launch finds its planes in the 256 MiB last-level cache, as in a pipeline that
+    # streams batches through the transform.  Set 0 is configs[1]'s own tensor (seed 1).
+    xs = [synth.normal((B, N, N), seed=1 + i, device=dev) for i in range(SETS)]
+    specs = [torch.empty((B, N // 2 + 1, N, 2), device=dev) for _ in range(SETS)]
+    x, spec = xs[0], specs[0]
+    back = torch.empty_like(x)
+    calls = [prepared("fbfft_r2c_2d", F, a, b, 0, 0) for a, b in zip(xs, specs)]
+    fwd = calls[0]
+    inv = prepared("fbfft_c2r_2d", F, spec, back, 0, 0)
+    turn = [0]
+
+    def step():
+        calls[turn[0] % SETS]()
+        turn[0] += 1
+
+    step_s, launch_s = timed(step, args.steps, args.warmup, torch)
+    launch_mid, launch_min = spread(step, args.steps, torch)
     value = nbytes / step_s / 1e9
 
     def hbm_roofline(nb, t, mid, low, note):
@@ -531,24 +641,51 @@ def main():
                 "launch_us": round(t * 1e6, 2), "launch_us_median": round(mid * 1e6, 2),
                 "launch_us_min": round(low * 1e6, 2), "residency": note}
 
-    # configs[1]'s 132 MB of operands fit the 256 MiB last-level cache when the same
-    # buffers are used launch after launch.  Two measurements whose operands come from
-    # HBM: the same 16384-plane launch rotating over four distinct buffer sets (528 MB),
-    # and one launch over a 4x batch.
-    sets = [(x, spec)]
-    for i in range(3):
-        sets.append((synth.normal((B, N, N), seed=100 + i, device=dev), torch.empty_like(spec)))
-    calls = [prepared("fbfft_r2c_2d", F, a, b, 0, 0) for a, b in sets]
-    turn = [0]
+    traffic, traffic_src = profile_traffic("fft2dSmallForward32_configs1.md",
+                                           "traffic_bytes_per_launch")
+    roofline = dict(hbm_roofline(nbytes, launch_s, launch_mid, launch_min,
+                                 "hbm: consecutive launches run on %d different sets of operands, "
+                                 "%d MB in all" % (SETS, SETS * nbytes // 1000000)),
+                    traffic=traffic, traffic_source=traffic_src)
 
-    def rotating():
-        calls[turn[0] & 3]()
+    # What moving the same bytes costs with no arithmetic, under the same rotation: the
+    # runtime's device-to-device copy and the library's own copy kernel, 66 MiB -> 66 MiB
+    # (configs[1] reads 64 MiB and writes 68 MiB).
+    half = nbytes // 2
+    csrc = [t.view(-1)[:half // 4] for t in specs]          # contents do not matter
+    cdst = [torch.empty(half // 4, device=dev) for _ in range(SETS)]
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    L = F.lib()
+
+    cargs = [(ctypes.c_void_p(a.data_ptr()), ctypes.c_void_p(b.data_ptr()), half, stream)
+             for a, b in zip(csrc, cdst)]
+
+    def copy_runtime():
+        i = turn[0] % SETS
         turn[0] += 1
-    _, rot_s = timed(rotating, max(args.steps, 40), max(args.warmup, 8), torch)
-    rot_mid, rot_min = spread(rotating, max(args.steps, 40), torch)
-    roofline_rotating = hbm_roofline(nbytes, rot_s, rot_mid, rot_min,
-                                     "hbm: configs[1] launches rotate over 4 buffer sets, 528 MB")
-    del sets, calls
+        cdst[i].copy_(csrc[i])
+
+    def copy_kernel():
+        i = turn[0] % SETS
+        turn[0] += 1
+        if L.fbfft_bench_copy(*cargs[i]) != 0:
+            raise RuntimeError("fbfft_bench_copy failed")
+    n_aux, w_aux = max(args.steps, 40), max(args.warmup, 8)
+    _, t_rt = timed(copy_runtime, n_aux, w_aux, torch)
+    _, t_ck = timed(copy_kernel, n_aux, w_aux, torch)
+    copy_ceiling = {
+        "bytes_per_launch": 2 * half, "residency": roofline["residency"],
+        "runtime_copy_us": round(t_rt * 1e6, 2), "runtime_copy_GBps": round(2 * half / t_rt / 1e9, 1),
+        "copy_kernel_us": round(t_ck * 1e6, 2), "copy_kernel_GBps": round(2 * half / t_ck / 1e9, 1),
+        "transform_over_copy_kernel": round(launch_s / t_ck, 3)}
+    del csrc, cdst, cargs
+
+    # the same launch on the same buffers over and over: operands in the last-level cache
+    _, llc_s = timed(fwd, max(args.steps, 200), max(args.warmup, 200), torch)
+    llc_mid, llc_min = spread(fwd, max(args.steps, 200), torch)
+    roofline_llc = hbm_roofline(nbytes, llc_s, llc_mid, llc_min,
+                                "last-level cache: the same 132 MB of operands every launch "
+                                "(not an HBM figure)")
     x4 = synth.normal((4 * B, N, N), seed=6, device=dev)
     s4 = torch.empty((4 * B, N // 2 + 1, N, 2), device=dev)
     f4 = prepared("fbfft_r2c_2d", F, x4, s4, 0, 0)
@@ -559,18 +696,31 @@ def main():
 
     extra = {}
     if not args.no_extra:
-        s, l = timed(inv, args.steps, args.warmup, torch)
+        # C2R and the packed-format pair, operands from HBM like the headline (the inverse of
+        # set i overwrites its own planes for i > 0; set 0 returns into `back`)
+        def rotate(cs):
+            def f():
+                cs[turn[0] % SETS]()
+                turn[0] += 1
+            return f
+        backs = [back] + xs[1:]
+        invs = [prepared("fbfft_c2r_2d", F, specs[i], backs[i], 0, 0) for i in range(SETS)]
+        _, l = timed(rotate(invs), n_aux, w_aux, torch)
+        extra["c2r_32x32_b16384_us"] = round(l * 1e6, 2)
         extra["c2r_32x32_b16384_GBps"] = round(nbytes / l / 1e9, 1)
         # round-trip sanity on the benchmark tensors themselves
         err = float((back / (N * N) - x).double().norm() / x.double().norm())
         extra["roundtrip_rel_l2"] = err
         # packed spectra of configs[1]: [B][16][32][2], 8192 bytes per plane
-        sp = torch.empty((B, N // 2, N, 2), device=dev)
-        _, lp = timed(prepared("fbfft_r2c_2d", F, x, sp, 0, 0), args.steps, args.warmup, torch)
-        _, lq = timed(prepared("fbfft_c2r_2d", F, sp, back, 0, 0), args.steps, args.warmup, torch)
+        sps = [t.view(-1)[:B * (N // 2) * N * 2].view(B, N // 2, N, 2) for t in specs]
+        pf = [prepared("fbfft_r2c_2d", F, backs[i] if i else x, sps[i], 0, 0) for i in range(SETS)]
+        pi = [prepared("fbfft_c2r_2d", F, sps[i], backs[i], 0, 0) for i in range(SETS)]
+        _, lp = timed(rotate(pf), n_aux, w_aux, torch)
+        _, lq = timed(rotate(pi), n_aux, w_aux, torch)
         extra["r2c_32x32_packed_b16384_GBps"] = round(B * 8192 / lp / 1e9, 1)
         extra["c2r_32x32_packed_b16384_GBps"] = round(B * 8192 / lq / 1e9, 1)
-        del sp
+        del sps, pf, pi, invs, backs
+        del xs[1:], specs[1:], calls
         for n2, b2 in ((16, 262144), (8, 1048576), (64, 16384), (128, 4096)):
             x2 = synth.normal((b2, n2, n2), seed=2 + n2.bit_length() - 1, device=dev)
             s2 = torch.empty((b2, n2 // 2 + 1, n2, 2), device=dev)
@@ -612,17 +762,19 @@ def main():
         "vs_baseline": None,
         "dtype": "f32",
         "data": "synthetic",
-        "config": {"workload": "configs[1]: fbfft2D R2C, 16384 planes of 32x32 fp32 N(0,1) seed 1, "
-                               "output [16384][17][32][2]; 8448 algorithmic bytes per plane"},
-        "roofline": dict(hbm_roofline(nbytes, launch_s, launch_mid, launch_min,
-                                      "last-level cache: the same 132 MB of operands every launch"),
-                         traffic=measured_traffic()),
-        "roofline_rotating": roofline_rotating,
+        "config": {"workload": "configs[1]: fbfft2D R2C, 16384 planes of 32x32 fp32 N(0,1), output "
+                               "[16384][17][32][2]; 8448 algorithmic bytes per plane; operands "
+                               "served from HBM (8 sets of buffers in turn, set 0 = seed 1)"},
+        "roofline": roofline,
+        "copy_ceiling": copy_ceiling,
+        "roofline_llc": roofline_llc,
         "roofline_4x": roofline_4x,
         "extra": extra,
     }
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(x.cpu().numpy(), N)
+        if not args.no_extra:
+            extra["fft_conv_cpu_baseline"] = conv_cpu_baseline()
     print(json.dumps(out))
 
 

@@ -51,7 +51,7 @@ EXPORTS = (
     "fbfft_make_tiles",
     "fbfft_make_tiles_for_pass",
     "fbfft_conv_choose_fft_size", "fbfft_conv_workspace", "fbfft_conv_workspace_image", "fbfft_conv_fprop_workspace", "fbfft_conv_fprop", "fbfft_conv_bprop",
-    "fbfft_conv_accgrad", "fbfft_conv_fprop_static", "fbfft_error_string",
+    "fbfft_conv_accgrad", "fbfft_conv_fprop_static", "fbfft_bench_copy", "fbfft_error_string",
     "fbfft_twiddle_table",
 )
 
@@ -103,6 +103,7 @@ def lib():
         L.fbfft_conv_accgrad.argtypes = [tp, tp, tp, ctypes.c_int, ctypes.c_float, ctypes.c_int, vp,
                                          ctypes.c_size_t, vp]
         L.fbfft_conv_fprop_static.argtypes = [tp, tp, tp, ctypes.c_int, vp]
+        L.fbfft_bench_copy.argtypes = [vp, vp, ctypes.c_size_t, vp]
         L.fbfft_error_string.argtypes = [ctypes.c_int]
         L.fbfft_error_string.restype = ctypes.c_char_p
         L.fbfft_twiddle_table.argtypes = [ctypes.POINTER(ctypes.c_float)]

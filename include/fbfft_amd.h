@@ -301,6 +301,13 @@ int fbfft_conv_accgrad(const fbfft_tensor* input, const fbfft_tensor* gradOutput
 int fbfft_conv_fprop_static(const fbfft_tensor* input, const fbfft_tensor* weight,
                             const fbfft_tensor* output, int fftSize, fbfft_stream_t stream);
 
+/* Measurement aid with no counterpart in the reference: a plain device-to-device copy
+ * of `bytes` (a multiple of 16, both pointers 16-byte aligned) on `stream`, in the
+ * shape that moves a batch the size of a transform's operands fastest from HBM to HBM.
+ * Benchmarks time it beside the transforms as the price of moving the same bytes with
+ * no arithmetic. */
+int fbfft_bench_copy(const void* src, void* dst, size_t bytes, fbfft_stream_t stream);
+
 /* Human-readable name of an fbfft_error. */
 const char* fbfft_error_string(int code);
 

@@ -265,6 +265,29 @@ def corr2d_grad_weight(inp, gout, kH, kW):
     return gw
 
 
+def corr2d_grad_input_at(gout, w, H, W, coords):
+    """fp64 gradInput of the valid correlation at the listed (n, c, y, x)."""
+    gout, w = _f32(gout), _f32(w)
+    Cout, Cin, kH, kW = w.shape
+    coords = np.ascontiguousarray(coords, dtype=np.int32)
+    out = np.zeros(len(coords), np.float64)
+    lib().ref64_corr2d_grad_input_at(_p(gout), _p(w), Cin, H, W, Cout, kH, kW, _p(coords),
+                                     len(coords), _p(out))
+    return out
+
+
+def corr2d_grad_weight_at(inp, gout, kH, kW, coords):
+    """fp64 gradWeight of the valid correlation at the listed (f, c, u, v)."""
+    inp, gout = _f32(inp), _f32(gout)
+    Nb, Cin, H, W = inp.shape
+    Cout = gout.shape[1]
+    coords = np.ascontiguousarray(coords, dtype=np.int32)
+    out = np.zeros(len(coords), np.float64)
+    lib().ref64_corr2d_grad_weight_at(_p(inp), _p(gout), Nb, Cin, H, W, Cout, kH, kW, _p(coords),
+                                      len(coords), _p(out))
+    return out
+
+
 def transpose_mm64(A, B, conjA, conjB, invNorm):
     A, B = _f32(A), _f32(B)
     XY = A.shape[2]

@@ -969,6 +969,48 @@ void ref64_corr2d_grad_weight(const float* in, const float* gout, int Nb, int Ci
         }
 }
 
+// The same two gradients restricted to lists of coordinates, so that layers too large for
+// the full sums can be spot-checked: (n, c, y, x) of gradInput, (f, c, u, v) of gradWeight.
+void ref64_corr2d_grad_input_at(const float* gout, const float* w, int Cin, int H, int W, int Cout,
+                                int kH, int kW, const int* coords, int ncoords, double* out) {
+  const int oH = H - kH + 1, oW = W - kW + 1;
+#pragma omp parallel for schedule(static)
+  for (int i = 0; i < ncoords; ++i) {
+    const int n = coords[4 * i], c = coords[4 * i + 1], y = coords[4 * i + 2], x = coords[4 * i + 3];
+    double acc = 0;
+    for (int f = 0; f < Cout; ++f)
+      for (int u = 0; u < kH; ++u) {
+        const int oy = y - u;
+        if (oy < 0 || oy >= oH) continue;
+        for (int v = 0; v < kW; ++v) {
+          const int ox = x - v;
+          if (ox < 0 || ox >= oW) continue;
+          acc += (double)gout[(((size_t)n * Cout + f) * oH + oy) * oW + ox] *
+                 (double)w[(((size_t)f * Cin + c) * kH + u) * kW + v];
+        }
+      }
+    out[i] = acc;
+  }
+}
+
+void ref64_corr2d_grad_weight_at(const float* in, const float* gout, int Nb, int Cin, int H, int W,
+                                 int Cout, int kH, int kW, const int* coords, int ncoords,
+                                 double* out) {
+  const int oH = H - kH + 1, oW = W - kW + 1;
+#pragma omp parallel for schedule(dynamic)
+  for (int i = 0; i < ncoords; ++i) {
+    const int f = coords[4 * i], c = coords[4 * i + 1], u = coords[4 * i + 2], v = coords[4 * i + 3];
+    double acc = 0;
+    for (int n = 0; n < Nb; ++n)
+      for (int y = 0; y < oH; ++y) {
+        const float* ir = in + (((size_t)n * Cin + c) * H + y + u) * W + v;
+        const float* gr = gout + (((size_t)n * Cout + f) * oH + y) * oW;
+        for (int x = 0; x < oW; ++x) acc += (double)ir[x] * (double)gr[x];
+      }
+    out[i] = acc;
+  }
+}
+
 // fp64 contraction with the transposeMM semantics (no invNorm on the
 // accumulated-into value: pure sum, scaled)
 void ref64_transpose_mm(const float* A, const float* B, double* C, int I, int J, int K, int XY,

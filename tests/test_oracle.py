@@ -259,6 +259,20 @@ def test_corr64_against_torch(oracle):
     coords = np.array([[0, 0, 0, 0], [1, 3, 6, 8], [1, 2, 3, 4]], np.int32)
     at = oracle.corr2d_valid_at(x, w, coords)
     assert np.allclose(at, [out[tuple(cc)].item() for cc in coords], rtol=1e-12)
+    # the subset forms of the two gradients: every element, against torch's autograd
+    # (borders, where part of the filter hangs over the edge of gradOutput, included)
+    gi_all = np.array([(n, ch, y, xx) for n in range(2) for ch in range(3) for y in range(9)
+                       for xx in range(10)], np.int32)
+    got = oracle.corr2d_grad_input_at(g, w, 9, 10, gi_all).reshape(2, 3, 9, 10)
+    assert rel(got, xt.grad.numpy()) < TOL64
+    gw_all = np.array([(f, ch, u, v) for f in range(4) for ch in range(3) for u in range(3)
+                       for v in range(2)], np.int32)
+    got = oracle.corr2d_grad_weight_at(x, g, 3, 2, gw_all).reshape(4, 3, 3, 2)
+    assert rel(got, wt.grad.numpy()) < TOL64
+    # a shuffled subset returns the same values in the order asked for
+    pick = rng.permutation(len(gi_all))[:17]
+    assert np.allclose(oracle.corr2d_grad_input_at(g, w, 9, 10, gi_all[pick]),
+                       xt.grad.numpy().reshape(-1)[pick], rtol=1e-12, atol=1e-14)
 
 
 def tiles_for(H, W, k, N):
