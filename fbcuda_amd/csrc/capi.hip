@@ -306,7 +306,11 @@ extern "C" int fbfft_conv_choose_fft_size(int pass, int batch, int cin, int cout
   for (int N = 8; N <= 32; N *= 2) {
     if (kH > N || kW > N) continue;
     const int spanY = pass == 1 ? H : H - kH + 1, spanX = pass == 1 ? W : W - kW + 1;
-    const double tiles = (double)((spanY + N - kH) / (N - kH + 1)) * ((spanX + N - kW) / (N - kW + 1));
+    // (an image that fits the transform is one window, whatever the pass: the rule of the
+    // launcher's own window grid)
+    const double tiles = (H <= N && W <= N)
+                             ? 1.0
+                             : (double)((spanY + N - kH) / (N - kH + 1)) * ((spanX + N - kW) / (N - kW + 1));
     const double values = (double)N * N * (tiles * batch * ((double)cin + cout) + (double)cin * cout);
     const double rate = N == 32 ? 1.0 : N == 16 ? (pass == 2 ? 1.25 : 1.15) : (pass == 2 ? 2.0 : 1.5);
     const double cost = values * rate;

@@ -285,7 +285,8 @@ __device__ __forceinline__ void forwardBinMajorBody(const ForwardJob& job, int w
 // LDS, and fly under the first run's transforms and stores.
 template <int N, bool ACC, int GROUPS, int PAIRS>
 __global__ __launch_bounds__(kTF) void inverseBinMajor(const float2* Cs, int I, int Jp, PlaneSet out,
-                                                       float scale, int splits, long splitStride) {
+                                                       float scale, int splits, long splitStride,
+                                                       int runGroups) {
   using C = BMCfg<N>;
   constexpr int H = C::H, T = C::T, SLOTS = C::SLOTS, RS = C::RS, PSZ = C::PSZ;
   constexpr int PER = C::BINS / T;
@@ -293,7 +294,9 @@ __global__ __launch_bounds__(kTF) void inverseBinMajor(const float2* Cs, int I, 
   __shared__ __align__(16) c32 lds[SLOTS * PSZ];
   const int t = threadIdx.x;
   const int s = t / T, l = t % T;
-  const int i = blockIdx.y;
+  // one grid index for (i, group of runs), runs fastest: a batch on i may exceed what a
+  // second grid dimension can count
+  const int i = blockIdx.x / runGroups, runGroup = blockIdx.x % runGroups;
   const int sp = t % SLOTS, bq = t / SLOTS;
   const long binStride = (long)I * Jp;
   c32* plane = lds + s * PSZ;
@@ -371,7 +374,7 @@ __global__ __launch_bounds__(kTF) void inverseBinMajor(const float2* Cs, int I, 
     }
   };
 
-  const int ja = blockIdx.x * GROUPS * SLOTS;
+  const int ja = runGroup * GROUPS * SLOTS;
   c32 in[PER];
   request(ja, in);
   park(in);
@@ -977,6 +980,12 @@ int runPipeline(PlaneSet x, PlaneSet y, PlaneSet out, bool conjY, float scale, b
   out.R = I;
   out.K = J;
   const int Ip = roundUp(I, SL), Jp = roundUp(J, SL), Kp = roundUp(K, 8);
+  // every launch below counts its workgroups in one 31-bit grid index: refuse, before
+  // anything runs, a layer whose transforms or contraction tiles outnumber that
+  const long gridMax = 0x7fffffffL;
+  if ((long)(Ip / SL + Jp / SL) * Kp > gridMax || (long)(Jp / SL) * I > gridMax ||
+      (long)bins * ceilDiv(I, 32) * ceilDiv(Jp, 32) > gridMax)
+    return FBFFT_UNSUPPORTED_SIZE;
   float2* SA = ws;
   float2* SB = SA + (size_t)bins * Kp * Ip;
   float2* SC = SB + (size_t)bins * Kp * Jp;
@@ -1048,7 +1057,8 @@ int runPipeline(PlaneSet x, PlaneSet y, PlaneSet out, bool conjY, float scale, b
   // 1936 paired workgroups; at configs[3] pairing would leave 768 workgroups, one and a
   // half rounds, and costs 35.5 -> 37.1 us.
   const bool pairedRuns = Jp / SL >= 2 && (long)ceilDiv(Jp / SL, 2) * I >= 3L * 2 * computeUnits();
-  const dim3 igrid(pairedRuns ? ceilDiv(Jp / SL, 2) : Jp / SL, I);
+  const int runGroups = pairedRuns ? ceilDiv(Jp / SL, 2) : Jp / SL;
+  const dim3 igrid((unsigned)((long)runGroups * I));
   // windows whose rows start on 8-byte boundaries with an even width: a lane stores its
   // two columns of a row as one 8-byte word
   const int po = movesAsPairs(out);
@@ -1056,7 +1066,8 @@ int runPipeline(PlaneSet x, PlaneSet y, PlaneSet out, bool conjY, float scale, b
   const float invNorm = 1.0f / (float)(N * N);
   auto launchInverse = [&](auto acc, auto groups, auto pairs) {
     inverseBinMajor<N, decltype(acc)::value, decltype(groups)::value, decltype(pairs)::value>
-        <<<igrid, dim3(kTF), 0, s>>>(SC, I, Jp, out, scale * invNorm, g.splits, g.splitStride);
+        <<<igrid, dim3(kTF), 0, s>>>(SC, I, Jp, out, scale * invNorm, g.splits, g.splitStride,
+                                     runGroups);
   };
   auto withPairs = [&](auto acc, auto groups) {
     if (po == 2)

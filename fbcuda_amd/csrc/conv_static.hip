@@ -12,6 +12,12 @@
 // on one stream are ordered.  Nothing in the array has to survive between calls
 // and nothing has to start at zero: the forward-transform kernels write every
 // element the contraction reads, padding rows included.
+//
+// The look-up happens in the first call on a device, whatever its operands - a call
+// with an empty batch does it and launches nothing - and may make the runtime load
+// this library's device image.  Callers that capture into a graph or must not
+// touch the allocator in their loop make that first call beforehand, outside
+// capture; later calls only enqueue kernels.
 #include "common.h"
 
 #include <atomic>
@@ -59,8 +65,8 @@ extern "C" int fbfft_conv_fprop_static(const fbfft_tensor* input, const fbfft_te
                                                  weight->size[3], fftSize);
   // need == 0: empty or unsupported shapes; fbfft_conv_fprop sorts those out and
   // never touches the workspace
-  if (need > (size_t)FBFFT_STATIC_SCRATCH_BYTES) return FBFFT_UNSUPPORTED_SIZE;
-  void* ws = scratchAddress();
+  void* ws = scratchAddress();  // before any other outcome: the first call is the set-up call
   if (!ws) return FBFFT_HIP_ERROR;
+  if (need > (size_t)FBFFT_STATIC_SCRATCH_BYTES) return FBFFT_UNSUPPORTED_SIZE;
   return fbfft_conv_fprop(input, weight, output, fftSize, ws, FBFFT_STATIC_SCRATCH_BYTES, stream);
 }

@@ -296,7 +296,11 @@ int fbfft_conv_accgrad(const fbfft_tensor* input, const fbfft_tensor* gradOutput
  * runs on holds its own copy until the process ends).  Layers whose
  * fbfft_conv_workspace(0, ...) exceeds that size return UnsupportedSize.  All
  * calls on one GPU share that GPU's array: calls on one stream are ordered, calls
- * that overlap in time on one GPU race.  Results are those of fbfft_conv_fprop. */
+ * that overlap in time on one GPU race.  Results are those of fbfft_conv_fprop.
+ * The first call on a device looks the array's address up (and may make the runtime
+ * load the library's device image); any call does, one with an empty batch included,
+ * which launches nothing.  Make that call before stream capture begins or before the
+ * loop that must not allocate; every later call only enqueues kernels. */
 #define FBFFT_STATIC_SCRATCH_BYTES (32u << 20)
 int fbfft_conv_fprop_static(const fbfft_tensor* input, const fbfft_tensor* weight,
                             const fbfft_tensor* output, int fftSize, fbfft_stream_t stream);

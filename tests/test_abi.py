@@ -263,6 +263,10 @@ def test_conv_choose_fft_size():
             # the workspace of size 0 is the workspace of the chosen size
             assert L.fbfft_conv_workspace_image(p, 4, 3, 5, H, W, kH, kW, 0) == \
                 L.fbfft_conv_workspace_image(p, 4, 3, 5, H, W, kH, kW, N) > 0
+    # an image that fits one 32-point window is one window for the input gradient too (its
+    # 30..32 rows are more than the 28 a window advances by, but there is nothing to advance to)
+    for H in (29, 30, 31, 32):
+        assert L.fbfft_conv_choose_fft_size(1, 128, 64, 192, H, H, 5, 5) == 32, H
     # no size holds the filter, the filter is larger than the image, bad pass or counts
     assert L.fbfft_conv_choose_fft_size(0, 4, 3, 5, 64, 64, 33, 3) == 0
     assert L.fbfft_conv_choose_fft_size(0, 4, 3, 5, 4, 4, 5, 5) == 0

@@ -469,3 +469,25 @@ def test_mm_random_aligned_shapes(oracle, seed):
                                B.reshape(B.shape[0], B.shape[1], xy, 2), conjA, conjB, 0.25,
                                C=C0.reshape(I, J, xy, 2) if acc else None)
     assert rel(got.reshape(I, J, xy, 2), want) < TOL_FFT, (I, J, K, shape, conjA, conjB, acc)
+
+
+def test_conv_fprop_batch_beyond_a_16_bit_grid_index(oracle):
+    """70000 images with 40 output planes keep the batch on the slow index of the product,
+    so the inverse transform's launch counts more than 65535 images: every image is
+    reached (whole tensor finite) and seeded pixels, the last images included, match."""
+    d = dev()
+    B, Cin, Cout, H, k, N = 70000, 2, 40, 8, 3, 8
+    x = synth.normal((B, Cin, H, H), seed=60, device=d)
+    w = synth.normal((Cout, Cin, k, k), seed=61, std=0.1, device=d)
+    out = torch.full((B, Cout, H - k + 1, H - k + 1), float("nan"), device=d)
+    assert F.conv_fprop(x, w, out, N, workspace(0, B, Cin, Cout, N)) == F.Success
+    torch.cuda.synchronize()
+    assert bool(torch.isfinite(out).all())
+    rng = np.random.default_rng(62)
+    coords = np.stack([rng.integers(0, B, 2048), rng.integers(0, Cout, 2048),
+                       rng.integers(0, H - k + 1, 2048), rng.integers(0, H - k + 1, 2048)],
+                      axis=1).astype(np.int32)
+    coords[:4, 0] = [0, 65535, 65536, B - 1]
+    want = oracle.corr2d_valid_at(x.cpu().numpy(), w.cpu().numpy(), coords)
+    oh = out.cpu().numpy()
+    assert rel(oh[coords[:, 0], coords[:, 1], coords[:, 2], coords[:, 3]], want) < TOL_CONV

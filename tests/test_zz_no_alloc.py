@@ -53,6 +53,49 @@ def test_static_scratch_matches_workspace_form(oracle):
     assert rel(out.cpu().numpy(), want64) < TOL_CONV
 
 
+def test_static_scratch_under_graph_capture_and_without_allocation():
+    """After one eager call (which looks the array up) the entry point can be captured into
+    a HIP graph, every replay equals the workspace form on the inputs of that moment, and
+    device memory in use is the same before and after the calls."""
+    d = dev()
+    B, Cin, Cout, H, W, k, N = 6, 10, 12, 27, 25, 5, 32
+    x, w = _layer(B, Cin, Cout, H, W, k, 60)
+    out = torch.full((B, Cout, H - k + 1, W - k + 1), float("nan"), device=d)
+    empty_x = torch.zeros((0, Cin, H, W), device=d)
+    empty_out = torch.zeros((0, Cout, H - k + 1, W - k + 1), device=d)
+    new_x = [synth.normal(tuple(x.shape), seed=70 + r).to(d) for r in range(3)]
+    torch.cuda.synchronize()
+    # the set-up call: an empty batch, nothing launched
+    assert F.conv_fprop_static(empty_x, w, empty_out, N) == F.Success
+    _with_workspace(x, w, N)   # the layer's kernels have run once: their code is resident
+    torch.cuda.synchronize()
+    free0, _ = torch.cuda.mem_get_info()
+    for _ in range(3):
+        assert F.conv_fprop_static(x, w, out, N) == F.Success
+    torch.cuda.synchronize()
+    free1, _ = torch.cuda.mem_get_info()
+    assert free1 == free0, "device memory in use changed across fbfft_conv_fprop_static"
+    want = _with_workspace(x, w, N)
+    assert torch.equal(out, want)
+
+    stream = torch.cuda.Stream()
+    stream.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(stream):
+        with torch.cuda.graph(graph, stream=stream):
+            assert F.conv_fprop_static(x, w, out, N, stream=stream) == F.Success
+    torch.cuda.synchronize()
+    for r in range(3):
+        x.copy_(new_x[r])
+        out.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        want = _with_workspace(x, w, N)   # eager work between the replays
+        assert bool(torch.isfinite(out).all())
+        assert torch.equal(out, want), "replay %d differs from the workspace form" % r
+
+
 def test_static_scratch_rejects_layers_beyond_its_size():
     B, Cin, Cout, N = 128, 64, 192, 32
     assert F.conv_fprop_workspace(B, Cin, Cout, N) > F.STATIC_SCRATCH_BYTES
