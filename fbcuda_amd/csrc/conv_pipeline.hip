@@ -172,6 +172,7 @@ struct ForwardJob {
   float imSign;
   int rowGroups;  // workgroups per k: Rp / SLOTS, or half of that (rounded up) when a
                   // workgroup takes two runs of rows
+  int stream;     // spectra leave with nontemporal stores
 };
 
 // Both operands of a pass in one launch: workgroups [0, a.rowGroups * a.Kp) transform
@@ -222,12 +223,17 @@ __device__ __forceinline__ void forwardBinMajorBody(const ForwardJob& job, int w
   // lanes: sp = t % SLOTS walks the run (consecutive rows), bq = t / SLOTS in [0, T)
   // walks bins: lane (sp, bq) stores columns x = bq and bq + T of every spectral row,
   // so LDS and HBM offsets are compile-time constants on top of one per-lane base.
-  auto copyOut = [&](int r0) __attribute__((always_inline)) {
+  auto copyOutAs = [&](int r0, auto streamTag) __attribute__((always_inline)) {
     const int sp = t % SLOTS, bq = t / SLOTS;
     const c32* src = lds + sp * PSZ + bq;
     const long binStride = (long)Kp * Rp;
     float2* dst = S + (long)k * Rp + r0 + sp + bq * binStride;
-    auto put = [&](int bin, c32 v) __attribute__((always_inline)) { dst[bin * binStride] = v; };
+    auto put = [&](int bin, c32 v) __attribute__((always_inline)) {
+      if constexpr (decltype(streamTag)::value)
+        streamStore(dst + bin * binStride, v);
+      else
+        dst[bin * binStride] = v;
+    };
     // Packed row 0 holds P[x] = F0[x] + i FH[x]: F0[x] = (P[x] + conj P[N-x]) / 2,
     // FH[x] = (P[x] - conj P[N-x]) / 2i.  Lane bq stores virtual bins bq (F0) and
     // T + bq (FH); bq = 0 stores the real pairs (F0[0], F0[N/2]) and (FH[0], FH[N/2]),
@@ -249,6 +255,17 @@ __device__ __forceinline__ void forwardBinMajorBody(const ForwardJob& job, int w
       put(r * N, c32{u.x, u.y * imSign});
       put(r * N + T, c32{v.x, v.y * imSign});
     });
+  };
+  // Spectra larger than the last-level cache can hold until the contraction reads them
+  // leave with the nontemporal hint (job.stream, the same for the whole launch): the
+  // weight gradient of a 16 x 32 x 256 x 256 layer in 1936 windows (2 x 254 MB of spectra)
+  // 310 -> 269 us; spectra that do fit (84 MB for 128 x 64 x 27 x 27 * 192 x 64 x 5 x 5)
+  // lose 2-7 % with it, because the contraction then fetches them from HBM.
+  auto copyOut = [&](int r0) __attribute__((always_inline)) {
+    if (job.stream)
+      copyOutAs(r0, std::true_type{});
+    else
+      copyOutAs(r0, std::false_type{});
   };
 
   const int ra = (wg % job.rowGroups) * GROUPS * SLOTS;
@@ -1003,8 +1020,10 @@ int runPipeline(PlaneSet x, PlaneSet y, PlaneSet out, bool conjY, float scale, b
   // times over (measured: 114.5 -> 109.8 us on 3936 workgroups, 29.9 -> 33.7 us on a
   // launch a quarter of that).
   const bool two = (long)(ceilDiv(Ip / SL, 2) + ceilDiv(Jp / SL, 2)) * Kp >= 3L * 2 * computeUnits();
-  const ForwardJob ja{x, SA, Ip, Kp, xSign, two ? ceilDiv(Ip / SL, 2) : Ip / SL},
-      jb{y, SB, Jp, Kp, ySign, two ? ceilDiv(Jp / SL, 2) : Jp / SL};
+  // both operands' spectra against half of the 256 MiB last-level cache
+  const int stream = (size_t)bins * Kp * ((size_t)Ip + Jp) * sizeof(float2) > (128u << 20);
+  const ForwardJob ja{x, SA, Ip, Kp, xSign, two ? ceilDiv(Ip / SL, 2) : Ip / SL, stream},
+      jb{y, SB, Jp, Kp, ySign, two ? ceilDiv(Jp / SL, 2) : Jp / SL, stream};
   const dim3 fgrid((unsigned)(ja.rowGroups + jb.rowGroups) * Kp);
   const int pa = movesAsPairs(x), pb = movesAsPairs(y);
   auto launchForward = [&](auto groups) {

@@ -399,7 +399,7 @@ __global__ __launch_bounds__(k1dThreads, 2) void fft1dMidInverse(const float* __
             return zrow[k];
         },
         zz);
-    difFFT<H, false>(zz);
+    regFFT<H, false>(zz);
     // private row, all of it in registers: store x[2j], x[2j+1]
     staticFor<Q>([&](auto jj) {
       constexpr int j = decltype(jj)::value;
@@ -443,7 +443,7 @@ __global__ __launch_bounds__(k1dThreads, 2) void fft1dMidInverse(const float* __
         pairFix(std::integral_constant<int, 4 * (Q - 1 - m) + 1>{}, drop, zz[m]);
       });
     }
-    difFFT<Q, false>(zz);
+    regFFT<Q, false>(zz);
     // w^(g j), w = e^(2 pi i / H); exponents of H/2 and more are the negated lower half
     auto twist = [&](auto gg) __attribute__((always_inline)) {
       constexpr int GG = decltype(gg)::value;
@@ -492,7 +492,7 @@ __global__ __launch_bounds__(k1dThreads, 2) void fft1dMidInverse(const float* __
         pairFix(std::integral_constant<int, k>{}, zz[(k - 1) / 2], zz[(H - k - 1) / 2]);
       });
     }
-    difFFT<Q, false>(zz);
+    regFFT<Q, false>(zz);
     if (g == 1) {
       staticFor<Q>([&](auto jj) {
         constexpr int j = decltype(jj)::value;

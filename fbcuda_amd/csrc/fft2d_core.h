@@ -197,8 +197,8 @@ template <int N, bool SPLIT = false>
 __device__ __forceinline__ void columnPassForward(c32 (&z0)[N / 2], c32 (&z1)[N / 2], c32* plane,
                                                   int l) {
   constexpr int H = N / 2, RS = PlaneCfg<N>::RS;
-  difFFT<H, true>(z0);
-  difFFT<H, true>(z1);
+  regFFT<H, true>(z0);
+  regFFT<H, true>(z1);
   c32 p0[H], p1[H];
   realFixupForward<H>(z0, p0);
   realFixupForward<H>(z1, p1);
@@ -230,7 +230,7 @@ __device__ __forceinline__ void rowPassInPlace(c32* plane, int l) {
     row[2 * j] = c32{v.x, v.y};
     row[2 * j + 1] = c32{v.z, v.w};
   });
-  difFFT<N, FWD>(row);
+  regFFT<N, FWD>(row);
   staticFor<N / 2>([&](auto jj) {
     constexpr int j = decltype(jj)::value;
     ldsStore4(p + 2 * j, row[slot<N>(2 * j)], row[slot<N>(2 * j + 1)]);
@@ -266,8 +266,8 @@ __device__ __forceinline__ void columnPassInverse(const c32* plane, int l, c32 (
   }
   realFixupInverse<H>(p0, z0);
   realFixupInverse<H>(p1, z1);
-  difFFT<H, false>(z0);
-  difFFT<H, false>(z1);
+  regFFT<H, false>(z0);
+  regFFT<H, false>(z1);
 }
 
 // Two columns of results through a bounds-checked strided view (crop on store).

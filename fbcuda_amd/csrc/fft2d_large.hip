@@ -167,7 +167,7 @@ __global__ __launch_bounds__(LargeCfg<N>::THREADS) void fft2dLargeForward(RealVi
     }
     __syncthreads();  // every row is in registers: the buffer may be overwritten
     if (t < N) {
-      difFFT<H, true>(z);
+      regFFT<H, true>(z);
       // ---- 3. fix-up fused with the transposed write: [kx][y] ----
       realFixupForwardEmit<H>(z, [&](auto kk, c32 val) {
         constexpr int k = decltype(kk)::value;
@@ -322,7 +322,7 @@ __global__ __launch_bounds__(LargeCfg<N>::THREADS) void fft2dLargeInverse(CplxVi
     {
       const c32* row = cb + t * YS;
       realFixupInverseFetch<H>([&](auto kk) { return row[decltype(kk)::value]; }, z);
-      difFFT<H, false>(z);
+      regFFT<H, false>(z);
     }
     __syncthreads();
     {
@@ -396,7 +396,7 @@ __global__ __launch_bounds__(LargeCfg<N>::THREADS) void fft2dLargeInverse(CplxVi
         });
       }
     }
-    difFFT<Q, false>(zz);
+    regFFT<Q, false>(zz);
     if (g == 1) {
       staticFor<Q>([&](auto jj) {
         constexpr int j = decltype(jj)::value;

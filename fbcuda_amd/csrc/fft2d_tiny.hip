@@ -26,7 +26,7 @@ __device__ __forceinline__ void forwardPlane(const float (&x)[N][N], c32 (&spec)
   staticFor<N>([&](auto yy) {
     constexpr int y = decltype(yy)::value;
     staticFor<N>([&](auto xx) { rows[y][decltype(xx)::value] = c32{x[y][decltype(xx)::value], 0.0f}; });
-    difFFT<N, true>(rows[y]);
+    regFFT<N, true>(rows[y]);
   });
   staticFor<N / 2 + 1>([&](auto kk) {
     constexpr int kx = decltype(kk)::value;
@@ -35,7 +35,7 @@ __device__ __forceinline__ void forwardPlane(const float (&x)[N][N], c32 (&spec)
       constexpr int y = decltype(yy)::value;
       col[y] = rows[y][slot<N>(kx)];
     });
-    difFFT<N, true>(col);
+    regFFT<N, true>(col);
     staticFor<N>([&](auto ff) {
       constexpr int ky = decltype(ff)::value;
       spec[kx][ky] = col[slot<N>(ky)];
@@ -52,7 +52,7 @@ __device__ __forceinline__ void inversePlane(const c32 (&spec)[N / 2 + 1][N], fl
     constexpr int kx = decltype(kk)::value;
     c32 col[N];
     staticFor<N>([&](auto ff) { col[decltype(ff)::value] = spec[kx][decltype(ff)::value]; });
-    difFFT<N, false>(col);
+    regFFT<N, false>(col);
     staticFor<N>([&](auto yy) {
       constexpr int y = decltype(yy)::value;
       g[kx][y] = col[slot<N>(y)];
@@ -69,7 +69,7 @@ __device__ __forceinline__ void inversePlane(const c32 (&spec)[N / 2 + 1][N], fl
       else
         row[kx] = cconj(g[N - kx][y]);
     });
-    difFFT<N, false>(row);
+    regFFT<N, false>(row);
     staticFor<N>([&](auto xx) {
       constexpr int xi = decltype(xx)::value;
       x[y][xi] = row[slot<N>(xi)].x;

@@ -60,7 +60,7 @@ __device__ __forceinline__ void splitFFT(const c32* col, int g, const c32* tw, c
       v[j] = cmul(comb, w);
     });
   }
-  difFFT<L, FWD>(v);
+  regFFT<L, FWD>(v);
 }
 
 }  // namespace fbfft_amd

@@ -96,28 +96,85 @@ __device__ __forceinline__ c32 mulHalfRoot(c32 d) {
   }
 }
 
-// Radix-2 decimation in frequency of a[0..N): natural order in, bit-reversed
-// order out (the value with frequency index k ends up in a[bitrev(k)]).
-template <int N, bool FWD, int M = N>
-__device__ __forceinline__ void difFFT(c32 (&a)[N]) {
-  if constexpr (M >= 2) {
-    constexpr int half = M / 2;
-    staticFor<N / M>([&](auto blk) {
-      staticFor<half>([&](auto kk) {
-        constexpr int k = decltype(kk)::value;
-        constexpr int lo = decltype(blk)::value * M + k;
-        constexpr int hi = lo + half;
-        c32 s = cadd(a[lo], a[hi]);
-        c32 d = csub(a[lo], a[hi]);
-        a[lo] = s;
-        a[hi] = mulRoot<M, k, FWD>(d);
-      });
-    });
-    difFFT<N, FWD, M / 2>(a);
+// One decimation-in-time butterfly with the twiddle folded into the additions:
+// (a, b) <- (a + W b, a - W b), W = e^{-/+ 2*pi*i*K/M} (forward: minus), K in [0, M/2).
+// A general W = c + i s costs six multiply-adds instead of the eight instructions of
+// "multiply, then add and subtract": with t = s / c, W b = c (b.x - t b.y, b.y + t b.x),
+// so two multiply-adds form the bracket and four more apply c while adding to a (the
+// bracket is taken relative to the larger of |c| and |s|, so |t| <= 1).  The roots on the
+// diagonals cost two additions and four multiply-adds, +-1 and +-i four additions.
+template <int M, int K, bool FWD>
+__device__ __forceinline__ void butterfly(c32& a, c32& b) {
+  static_assert(K >= 0 && 2 * K < M, "root index");
+  const c32 p = a, q = b;
+  if constexpr (K == 0) {
+    a = cadd(p, q);
+    b = csub(p, q);
+  } else if constexpr (4 * K == M) {  // W = -i (forward), +i (inverse)
+    if constexpr (FWD) {
+      a = c32{p.x + q.y, p.y - q.x};
+      b = c32{p.x - q.y, p.y + q.x};
+    } else {
+      a = c32{p.x - q.y, p.y + q.x};
+      b = c32{p.x + q.y, p.y - q.x};
+    }
+  } else if constexpr (8 * K == M || 8 * K == 3 * M) {
+    constexpr float h = TableEntry<32>::c;  // sqrt(1/2)
+    // W q = h (u, v)
+    float u, v;
+    if constexpr (8 * K == M) {
+      u = FWD ? q.x + q.y : q.x - q.y;
+      v = FWD ? q.y - q.x : q.x + q.y;
+    } else {
+      u = FWD ? q.y - q.x : -(q.x + q.y);
+      v = FWD ? -(q.x + q.y) : q.x - q.y;
+    }
+    a = c32{__builtin_fmaf(h, u, p.x), __builtin_fmaf(h, v, p.y)};
+    b = c32{__builtin_fmaf(-h, u, p.x), __builtin_fmaf(-h, v, p.y)};
+  } else {
+    constexpr float c = TableEntry<K * 256 / M>::c;
+    constexpr float s = FWD ? -TableEntry<K * 256 / M>::s : TableEntry<K * 256 / M>::s;
+    constexpr bool byCos = (c < 0 ? -c : c) >= (s < 0 ? -s : s);
+    if constexpr (byCos) {
+      constexpr float t = (float)((double)s / (double)c);
+      const float u = __builtin_fmaf(-t, q.y, q.x), v = __builtin_fmaf(t, q.x, q.y);
+      a = c32{__builtin_fmaf(c, u, p.x), __builtin_fmaf(c, v, p.y)};
+      b = c32{__builtin_fmaf(-c, u, p.x), __builtin_fmaf(-c, v, p.y)};
+    } else {
+      // W q = s (t q.x - q.y, q.x + t q.y), t = c / s
+      constexpr float t = (float)((double)c / (double)s);
+      const float u = __builtin_fmaf(t, q.x, -q.y), v = __builtin_fmaf(t, q.y, q.x);
+      a = c32{__builtin_fmaf(s, u, p.x), __builtin_fmaf(s, v, p.y)};
+      b = c32{__builtin_fmaf(-s, u, p.x), __builtin_fmaf(-s, v, p.y)};
+    }
   }
 }
 
-// index of frequency k in the output of difFFT<N>
+// In-register FFT of a[0..N): natural order in, bit-reversed order out (the value with
+// frequency index k ends up in a[bitrev(k)] = a[slot<N>(k)]).  Radix-2 decimation in
+// time run on renamed registers: logical position i of the textbook algorithm
+// (bit-reversed input, natural output) is register a[bitrev(i)], so the caller's
+// natural-order input is already in place and the output lands where a decimation in
+// frequency would have left it.  32 points: 388 vector instructions where the
+// decimation-in-frequency form (add, subtract, then multiply) took 456.
+template <int N, bool FWD, int M = 2>
+__device__ __forceinline__ void regFFT(c32 (&a)[N]) {
+  if constexpr (M <= N) {
+    constexpr int half = M / 2;
+    constexpr int bits = ilog2(N);
+    staticFor<N / M>([&](auto blk) {
+      staticFor<half>([&](auto kk) {
+        constexpr int k = decltype(kk)::value;
+        constexpr int lo = bitrev(decltype(blk)::value * M + k, bits);
+        constexpr int hi = bitrev(decltype(blk)::value * M + k + half, bits);
+        butterfly<M, k, FWD>(a[lo], a[hi]);
+      });
+    });
+    regFFT<N, FWD, 2 * M>(a);
+  }
+}
+
+// index of frequency k in the output of regFFT<N>
 template <int N>
 constexpr int slot(int k) {
   return bitrev(k, ilog2(N));
@@ -137,7 +194,7 @@ __device__ __forceinline__ void realPairForward(c32 a, c32 b, c32& fk, c32& fhk)
   fhk = c32{__builtin_fmaf(0.5f, e2.x, -t.x), __builtin_fmaf(-0.5f, e2.y, t.y)};
 }
 
-// Forward real-input fix-up.  z (in difFFT output order) is the H-point complex
+// Forward real-input fix-up.  z (in regFFT output order) is the H-point complex
 // FFT of z[j] = x[2j] + i*x[2j+1].  emit(k, value) is called once for every
 // k = 0..H-1 (k as an integral_constant) with F[k] of the 2H-point real
 // transform; for k = 0 the value is (F[0], F[H]) packed as (re, im) - both are
