@@ -454,16 +454,23 @@ def conv_extras(F, synth, torch, dev, extra):
 
 def run_only(name, steps, warmup, F, synth, torch, dev):
     """One workload in a tight loop, for profiling."""
-    if name in ("r2c32", "c2r32", "r2c64", "c2r64", "r2c128", "c2r128"):
-        n = int(name[3:])
-        b = int(os.environ.get("FBFFT_BENCH_B", {32: 16384, 64: 16384, 128: 4096}[n]))
+    import re
+    m2 = re.fullmatch(r"(r2c|c2r)(8|16|32|64|128)", name)
+    if m2:
+        # one 2D size on one set of buffers: configs[2]'s batches (256 MiB of input, far beyond
+        # the last-level cache) and configs[1]'s 16384 planes at 32 x 32 (which stay in it:
+        # r2c32hbm / c2r32hbm are the forms that read from HBM)
+        n = int(m2.group(2))
+        b = int(os.environ.get("FBFFT_BENCH_B", {8: 1 << 20, 16: 1 << 18, 32: 16384, 64: 16384,
+                                                 128: 4096}[n]))
         x = synth.normal((b, n, n), seed=1, device=dev)
         spec = torch.empty((b, n // 2 + 1, n, 2), device=dev)
         fwd = prepared("fbfft_r2c_2d", F, x, spec, 0, 0)
         fwd()
         fn = fwd if name.startswith("r2c") else prepared("fbfft_c2r_2d", F, spec, x, 0, 0)
         _, t = timed(fn, steps, warmup, torch)
-        return {"only": name, "us": round(t * 1e6, 2), "GBps": round(b * plane_bytes(n) / t / 1e9, 1)}
+        return {"only": name, "planes": b, "us": round(t * 1e6, 2),
+                "GBps": round(b * plane_bytes(n) / t / 1e9, 1)}
     if name in ("r2c32hbm", "c2r32hbm"):
         # configs[1] with operands served from HBM: eight sets of buffers in turn
         n, b, sets = 32, 16384, 8
@@ -481,15 +488,18 @@ def run_only(name, steps, warmup, F, synth, torch, dev):
             turn[0] += 1
         _, t = timed(step, steps, warmup, torch)
         return {"only": name, "us": round(t * 1e6, 2), "GBps": round(b * plane_bytes(n) / t / 1e9, 1)}
-    if name in ("r2c1d", "c2r1d"):
-        n, b = 256, 1 << 18
+    m1 = re.fullmatch(r"(r2c|c2r)1d(32|64|128|256)?", name)
+    if m1:
+        # 1D: configs[0] (32 points, 4096 rows) or 256 MiB of input at the larger sizes
+        n = int(m1.group(2) or 256)
+        b = 4096 if n == 32 else (1 << 26) // n
         x = synth.uniform((b, n), seed=0, device=dev)
         spec = torch.empty((b, n // 2 + 1, 2), device=dev)
         fwd = prepared("fbfft_r2c_1d", F, x, spec, 0)
         fwd()
-        fn = fwd if name == "r2c1d" else prepared("fbfft_c2r_1d", F, x, spec, 0)
+        fn = fwd if m1.group(1) == "r2c" else prepared("fbfft_c2r_1d", F, x, spec, 0)
         _, t = timed(fn, steps, warmup, torch)
-        return {"only": name, "us": round(t * 1e6, 2),
+        return {"only": name, "rows": b, "us": round(t * 1e6, 2),
                 "GBps": round(b * (4 * n + 8 * (n // 2 + 1)) / t / 1e9, 1)}
     extra = {}
     if name in ("iter4", "iter4ws"):
@@ -574,9 +584,11 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the informative extra configs")
     ap.add_argument("--only", default=None,
-                    choices=["r2c32hbm", "c2r32hbm", "r2c32", "c2r32", "r2c64", "c2r64", "r2c128", "c2r128", "mm", "conv",
-                             "conv_bprop", "conv_accgrad", "iterconv", "iter4", "iter4ws", "conv4",
-                             "conv4_bprop", "conv4_accgrad", "r2c1d", "c2r1d"],
+                    choices=["r2c32hbm", "c2r32hbm"] +
+                            [d + n for d in ("r2c", "c2r") for n in ("8", "16", "32", "64", "128")] +
+                            [d + "1d" + n for d in ("r2c", "c2r") for n in ("", "32", "64", "128", "256")] +
+                            ["mm", "conv", "conv_bprop", "conv_accgrad", "iterconv", "iter4", "iter4ws",
+                             "conv4", "conv4_bprop", "conv4_accgrad"],
                     help="run just this workload --steps times (for rocprofv3) and print its timing")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="only run a plain 256 MiB device-to-device copy 20 times: the known-size "
