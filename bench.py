@@ -547,7 +547,8 @@ def run_only(name, steps, warmup, F, synth, torch, dev):
             w = synth.normal((cout, cin, k, k), seed=41, std=0.05, device=dev)
         else:
             nb = int(os.environ.get("FBFFT_BENCH_CONV_B", "128"))  # profiling aid: other batch sizes
-            cin, cout, hw, k = 64, 192, 27, 5
+            cin, cout, k = 64, 192, 5
+            hw = int(os.environ.get("FBFFT_BENCH_CONV_HW", "27"))  # profiling aid: other image sizes
             x = synth.normal((nb, cin, hw, hw), seed=30, device=dev)
             w = synth.normal((cout, cin, k, k), seed=31, std=0.02, device=dev)
         o = synth.normal((nb, cout, hw - k + 1, hw - k + 1), seed=32, device=dev)

@@ -25,6 +25,15 @@ def rel(a, b):
     return float(np.linalg.norm(a - b) / max(np.linalg.norm(b), 1e-300))
 
 
+def check(label, got, want, tol):
+    """Asserts rel-L2(got, want) < tol and prints the observed figure (`pytest -s` shows it:
+    the parity numbers quoted in the documents come from these lines)."""
+    e = rel(got, want)
+    print("parity %-58s rel-L2 %.2e (bar %.0e)" % (label, e, tol))
+    assert e < tol, "%s: rel-L2 %.3e >= %.0e" % (label, e, tol)
+    return e
+
+
 def fft2d(x, N, padL=0, padU=0):
     """numpy real [B][h][w] -> numpy [B][N/2+1][N][2] through the C ABI."""
     xd = torch.from_numpy(np.ascontiguousarray(x, dtype=np.float32)).to(dev())

@@ -9,7 +9,7 @@ import torch
 
 import fbcuda_amd as F
 from fbcuda_amd import synth
-from gpu_util import TOL_CONV, dev, rel
+from gpu_util import check, TOL_CONV, dev, rel
 
 pytestmark = pytest.mark.gpu
 
@@ -120,7 +120,7 @@ def test_config4_through_the_layer_entry_point(oracle):
     want = oracle.corr2d_valid_at(x.cpu().numpy(), w.cpu().numpy(), coords)
     oh = out.cpu().numpy()
     got = oh[coords[:, 0], coords[:, 1], coords[:, 2], coords[:, 3]]
-    assert rel(got, want) < TOL_CONV
+    check("configs[4] fbfft_conv_fprop vs fp64 (4096 pixels)", got, want, TOL_CONV)
 
 
 @pytest.mark.parametrize("H,W,k", [(60, 60, 5), (14, 12, 3), (8, 8, 3), (27, 27, 5)])

@@ -7,7 +7,7 @@ import torch
 
 import fbcuda_amd as F
 from fbcuda_amd import synth
-from gpu_util import TOL_FFT, c, dev, rel
+from gpu_util import check, TOL_FFT, c, dev, rel
 
 pytestmark = pytest.mark.gpu
 GOLD = np.load(os.path.join(os.path.dirname(__file__), "golden", "fft_vectors.npz"))
@@ -61,10 +61,10 @@ def test_config0_full(oracle):
     rc, got = fft1d(x)
     assert rc == F.Success and got.shape == (4096, 17, 2)
     _, want = oracle.fbfft1d(x)
-    assert rel(got, want) < TOL_FFT
-    assert rel(got, oracle.dft1d_r2c(x)) < TOL_FFT
+    check("configs[0] fbfft1D vs transcription (4096 rows)", got, want, TOL_FFT)
+    check("configs[0] fbfft1D vs fp64 DFT", got, oracle.dft1d_r2c(x), TOL_FFT)
     rc, back = ifft1d(got)
-    assert rel(back, 32 * x.astype(np.float64)) < TOL_FFT
+    check("configs[0] round trip", back, 32 * x.astype(np.float64), TOL_FFT)
 
 
 @pytest.mark.parametrize("N", [4, 16, 32, 128])

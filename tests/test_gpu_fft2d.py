@@ -9,7 +9,7 @@ import torch
 
 import fbcuda_amd as F
 from fbcuda_amd import synth
-from gpu_util import TOL_FFT, c, dev, fft2d, ifft2d, rel
+from gpu_util import TOL_FFT, c, check, dev, fft2d, ifft2d, rel
 
 pytestmark = pytest.mark.gpu
 GOLD = np.load(os.path.join(os.path.dirname(__file__), "golden", "fft_vectors.npz"))
@@ -134,6 +134,7 @@ def test_full_size_properties(oracle, N, B):
     assert F.fbifft2D(spec, back) == F.Success
     torch.cuda.synchronize()
     err = (back / (N * N) - x).double().norm() / x.double().norm()
+    print("parity round trip %dx%d over all %d planes: %.2e" % (N, N, B, float(err)))
     assert float(err) < TOL_FFT
     if N == 32:
         pick = np.arange(B)
@@ -144,8 +145,12 @@ def test_full_size_properties(oracle, N, B):
     rc, want = oracle.fbfft2d(xp, N)
     assert rc == 0
     got = spec.cpu().numpy()[pick]
-    assert rel(got, want) < TOL_FFT
-    assert per_plane_rel(got, want) < TOL_FFT
+    tag = "%dx%d, %d of %d planes" % (N, N, len(pick), B)
+    check("fbfft2D vs transcription (%s)" % tag, got, want, TOL_FFT)
+    check("fbfft2D vs fp64 DFT (first 64 of them)", got[:64], oracle.dft2d_r2c(xp[:64], N), TOL_FFT)
+    worst = per_plane_rel(got, want)
+    print("parity fbfft2D worst single plane (%s): %.2e" % (tag, worst))
+    assert worst < TOL_FFT
     # inverse: the same spectra (the transcription's) into both implementations
     rc, want_back = oracle.fbifft2d(want, N, N)
     assert rc == 0
@@ -153,7 +158,7 @@ def test_full_size_properties(oracle, N, B):
     bd = torch.full((len(pick), N, N), float("nan"), device=d)
     assert F.fbifft2D(sd, bd) == F.Success
     torch.cuda.synchronize()
-    assert rel(bd.cpu().numpy(), want_back) < TOL_FFT
+    check("fbifft2D vs transcription, same spectra (%s)" % tag, bd.cpu().numpy(), want_back, TOL_FFT)
     assert per_plane_rel(bd.cpu().numpy(), want_back) < TOL_FFT
     del sd, bd
     # linearity on a slice: F(2x + y) = 2F(x) + F(y)

@@ -9,7 +9,7 @@ import torch
 
 import fbcuda_amd as F
 from fbcuda_amd import synth
-from gpu_util import TOL_CONV, dev, rel
+from gpu_util import TOL_CONV, check, dev, rel
 
 pytestmark = pytest.mark.gpu
 
@@ -55,9 +55,11 @@ def test_config3_gradients_through_the_layer_entry_points(oracle):
     rng = np.random.default_rng(35)
     ci = grad_input_coords(rng, 128, 64, 27, 27, 4096,
                            [[0, 0], [26, 26], [0, 26], [26, 0], [4, 4], [22, 22], [3, 23], [13, 0]])
-    assert rel(at(gi, ci), oracle.corr2d_grad_input_at(gh, wh, 27, 27, ci)) < TOL_CONV
+    check("configs[3] fbfft_conv_bprop vs fp64 (4096 elements)", at(gi, ci),
+          oracle.corr2d_grad_input_at(gh, wh, 27, 27, ci), TOL_CONV)
     cw = grad_weight_coords(rng, 192, 64, 5, 512)
-    assert rel(at(gw, cw), oracle.corr2d_grad_weight_at(xh, gh, 5, 5, cw)) < TOL_CONV
+    check("configs[3] fbfft_conv_accgrad vs fp64 (512 elements)", at(gw, cw),
+          oracle.corr2d_grad_weight_at(xh, gh, 5, 5, cw), TOL_CONV)
 
 
 @pytest.fixture(scope="module")
@@ -95,8 +97,8 @@ def test_config4_gradients_through_the_layer_entry_points(config4, config4_refer
                           ws_bytes(F.conv_workspace_image(2, 16, 32, 32, 256, 256, 9, 9, 32))) == F.Success
     torch.cuda.synchronize()
     assert bool(torch.isfinite(gi).all()) and bool(torch.isfinite(gw).all())
-    assert rel(at(gi, ci), want_i) < TOL_CONV
-    assert rel(at(gw, cw), want_w) < TOL_CONV
+    check("configs[4] fbfft_conv_bprop vs fp64 (4096 elements)", at(gi, ci), want_i, TOL_CONV)
+    check("configs[4] fbfft_conv_accgrad vs fp64 (256 elements)", at(gw, cw), want_w, TOL_CONV)
 
 
 @pytest.mark.parametrize("route", ["fused", "workspace"])
@@ -121,11 +123,11 @@ def test_config4_gradients_through_the_tile_descriptors(config4, config4_referen
     assert nb == 121
     assert run(bins, bouts, w, F.FFT_UpdateGradInput, nb)
     assert bool(torch.isfinite(gi).all())
-    assert rel(at(gi, ci), want_i) < TOL_CONV
+    check("configs[4] updateGradInput, %s route, vs fp64" % route, at(gi, ci), want_i, TOL_CONV)
 
     gw = torch.full_like(w, float("nan"))
     ins, outs, n = F.make_tile_grid(x, g, 9, 9, 32)
     assert n == 121
     assert run(ins, outs, gw, F.FFT_AccGradParameters, n)
     assert bool(torch.isfinite(gw).all())
-    assert rel(at(gw, cw), want_w) < TOL_CONV
+    check("configs[4] accGradParameters, %s route, vs fp64" % route, at(gw, cw), want_w, TOL_CONV)

@@ -7,7 +7,7 @@ import torch
 
 import fbcuda_amd as F
 from fbcuda_amd import synth
-from gpu_util import TOL_CONV, dev, rel
+from gpu_util import check, TOL_CONV, dev, rel
 
 pytestmark = pytest.mark.gpu
 
@@ -155,7 +155,7 @@ def test_config4_forward(oracle):
     want = oracle.corr2d_valid_at(x.cpu().numpy(), w.cpu().numpy(), coords)
     oh = out.cpu().numpy()
     got = oh[coords[:, 0], coords[:, 1], coords[:, 2], coords[:, 3]]
-    assert rel(got, want) < TOL_CONV
+    check("configs[4] FFTIteratedConvolution updateOutput vs fp64 (4096 pixels)", got, want, TOL_CONV)
 
 
 def test_library_tile_grid_matches_reference_tiling(oracle):

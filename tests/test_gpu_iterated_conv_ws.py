@@ -9,7 +9,7 @@ import torch
 
 import fbcuda_amd as F
 from fbcuda_amd import synth
-from gpu_util import TOL_CONV, dev, rel
+from gpu_util import check, TOL_CONV, dev, rel
 from test_gpu_iterated_conv import tiles_for
 
 pytestmark = pytest.mark.gpu
@@ -199,4 +199,5 @@ def test_config4_forward_through_the_workspace(oracle):
     coords[:8, 2:] = [[0, 0], [247, 247], [23, 24], [24, 23], [239, 240], [240, 239], [0, 247], [247, 0]]
     want = oracle.corr2d_valid_at(x.cpu().numpy(), w.cpu().numpy(), coords)
     oh = out.cpu().numpy()
-    assert rel(oh[coords[:, 0], coords[:, 1], coords[:, 2], coords[:, 3]], want) < TOL_CONV
+    check("configs[4] fbfft_iterated_conv_ws updateOutput vs fp64 (4096 pixels)",
+          oh[coords[:, 0], coords[:, 1], coords[:, 2], coords[:, 3]], want, TOL_CONV)

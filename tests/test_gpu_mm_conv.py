@@ -6,7 +6,7 @@ import torch
 
 import fbcuda_amd as F
 from fbcuda_amd import synth
-from gpu_util import TOL_CONV, TOL_FFT, dev, rel
+from gpu_util import check, TOL_CONV, TOL_FFT, dev, rel
 
 pytestmark = pytest.mark.gpu
 
@@ -177,7 +177,7 @@ def test_conv_fprop_config3(oracle):
     xh, wh, oh = x.cpu().numpy(), w.cpu().numpy(), out.cpu().numpy()
     want = oracle.corr2d_valid_at(xh, wh, coords)
     got = oh[coords[:, 0], coords[:, 1], coords[:, 2], coords[:, 3]]
-    assert rel(got, want) < TOL_CONV
+    check("configs[3] fbfft_conv_fprop vs fp64 (4096 pixels)", got, want, TOL_CONV)
     full = oracle.corr2d_valid(xh[[0, 127]], wh[[0, 191]])
     assert rel(oh[[0, 127]][:, [0, 191]], full) < TOL_CONV
 
