@@ -198,7 +198,14 @@ def conv_cpu_baseline(budget_s=12.0):
     ref = float(np.sum(x[0].astype(np.float64) [:, 3:8, 4:9] * w[5].astype(np.float64)))
     got = float(out.reshape(nb, cout, 23, 23)[0, 5, 3, 4])
     ms = (tw + tx * 128.0 / nb) * 1e3
+    # one thread, a slice of the batch, for scale
+    O.set_num_threads(1)
+    n1 = max(1, min(nb, 8))
+    tw1, tx1, _ = run(x[:n1])
+    O.set_num_threads(threads)
+    ms1 = (tw1 + tx1 * 128.0 / n1) * 1e3
     return {"value": round(ms, 1), "unit": "ms/iter", "cores": threads, "kind": "port",
+            "single_thread_ms_per_iter": round(ms1, 1),
             "sample": "%d pass(es) over %d of the 128 images of configs[3] with all 192x64 filters "
                       "(%.2f s for the image-dependent part, %.3f s for the filter transforms per "
                       "pass), scaled to 128 images" % (reps, nb, tx, tw),
