@@ -307,3 +307,25 @@ def test_empty_window_gives_zero_spectra(N, h, w):
     assert F.fbfft2D(x, out) == F.Success
     torch.cuda.synchronize()
     assert float(out.abs().max()) == 0.0
+
+
+@pytest.mark.parametrize("N,B", [(32, 8195), (32, 12289), (32, 14336), (32, 14339), (16, 30727),
+                                 (16, 53760), (16, 53767), (8, 98317), (8, 172032), (8, 172049)])
+def test_batches_either_side_of_the_two_groups_per_wave_switch(oracle, N, B):
+    """Batches just above one round of resident waves, at 1.75 rounds (the last that pair)
+    and just beyond (one group per wave again), odd tails included: every plane of the
+    forward transform against the transcription, and the inverse on its spectra."""
+    d = dev()
+    x = synth.normal((B, N, N), seed=70 + N, device=d)
+    spec = torch.full((B, N // 2 + 1, N, 2), float("nan"), device=d)
+    assert F.fbfft2D(x, spec) == F.Success
+    back = torch.full_like(x, float("nan"))
+    assert F.fbifft2D(spec, back) == F.Success
+    torch.cuda.synchronize()
+    rc, want = oracle.fbfft2d(x.cpu().numpy(), N)
+    assert rc == 0
+    got = spec.cpu().numpy()
+    assert np.isfinite(got).all()
+    assert per_plane_rel(got, want) < TOL_FFT
+    err = (back / (N * N) - x).double().norm() / x.double().norm()
+    assert bool(torch.isfinite(back).all()) and float(err) < TOL_FFT
