@@ -105,6 +105,18 @@ def test_cpp_device_tensor_and_complex_host_arithmetic():
     assert out.returncode == 0 and out.stdout.strip() == "OK", out.stdout
 
 
+def test_cpp_in_register_transforms_on_the_host():
+    """tests/cpp/regs_check.cpp: the butterfly and real-fix-up templates the kernels
+    instantiate (fbcuda_amd/csrc/fft_regs.h), compiled for the host and compared with a
+    naive fp64 DFT for 2 ... 128 complex points, both directions, and 4 ... 128 real points."""
+    import subprocess
+    subprocess.check_call(["make", "-C", os.path.join(ROOT, "tests", "cpp"), "-B", "regs_check"],
+                          stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL)
+    out = subprocess.run([os.path.join(ROOT, "tests", "cpp", "regs_check")], capture_output=True,
+                         text=True)
+    assert out.returncode == 0 and out.stdout.strip() == "OK", out.stdout
+
+
 def _fake_tensor(shape, base=0x10000000):
     """fbfft_tensor over memory that is never touched: the tile builder only does
     address arithmetic."""
