@@ -1,10 +1,11 @@
 // A plain device-to-device copy kernel, exported as a measurement aid: the yardstick
 // that the transform kernels' time per launch is held against (same bytes, no
 // arithmetic).  Each wave moves 16 KB: sixteen 16-byte loads per lane, all issued
-// before the first store, stores with the nontemporal hint - the fastest of the
-// shapes tried for a 66 MiB copy whose operands come from HBM (25.0 us; one 16-byte
-// word per lane 26.0 us, 4 per lane 28.3, 32 per lane 31.3, the runtime's own copy
-// 28.0 us).
+// before the first store, loads and stores with the nontemporal hint - the fastest of
+// the shapes tried for a 66 MiB copy whose operands come from HBM (24.9-25.0 us; the
+// same with plain loads 26.1-26.5 us, one 16-byte word per lane 25.6-26.0 us, 4 per lane
+// 27.8-28.3, 32 per lane 30.7-31.3, the runtime's own copy 28.0 us).  (For the
+// transforms themselves the hint pays on the stores only: on their loads it costs 5 %.)
 #include "common.h"
 
 namespace fbfft_amd {
@@ -19,7 +20,7 @@ __global__ __launch_bounds__(64) void benchCopyKernel(const vfloat4* __restrict_
 #pragma unroll
   for (int u = 0; u < kCopyWords; ++u) {
     const long i = base + 64 * u;
-    if (i < words) r[u] = src[i];
+    if (i < words) r[u] = __builtin_nontemporal_load(src + i);
   }
 #pragma unroll
   for (int u = 0; u < kCopyWords; ++u) {
